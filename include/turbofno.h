@@ -1,0 +1,98 @@
+/*
+ * turbofno.h -- C ABI of the MI355X (gfx950) implementation of TurboFNO's fused spectral layer
+ * (variant D, 1D and 2D): forward C2C FFT -> keep the 64 lowest modes -> complex GEMM over the
+ * channel dimension -> zero-pad -> backward FFT.
+ *
+ * The reference has no library API; its boundary is "host main() launches a __global__ kernel picked
+ * from a table indexed by log2(len)-7". Each entry point below replaces one such table entry and
+ * keeps its argument meaning. Reference paths are relative to the TurboFNO checkout.
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers to complex64 (interleaved float re, im). The caller owns
+ *     every buffer; the library allocates nothing and never synchronises the device.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Calls are asynchronous.
+ *   - Return value 0 = success; otherwise a TURBOFNO_ERR_* code, with a human-readable explanation
+ *     available from turbofno_last_error_string() (thread local). The library never exits the process
+ *     (the reference exits from its mains via CHECK_CUDA_KERNEL, utils/utils.cuh:17-25).
+ *   - 64 modes are retained per transformed axis (fused.cu:105, README.md:90); forward transforms use
+ *     exp(-2 pi i jm/D), backward transforms exp(+2 pi i jm/D) and are UNNORMALISED.
+ *   - Layouts: x[K][S][DY] (signal (k,s) at (k*S+s)*DY), W[k + n*K], y[N][S][DY]; in 2D
+ *     x[K][bs][DX][DY], y[N][bs][DX][DY].
+ */
+#ifndef TURBOFNO_H
+#define TURBOFNO_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TURBOFNO_OK               0
+#define TURBOFNO_ERR_INVALID_ARG  1  /* null pointer, non-positive size, K % 8, N % 64, M % 64 ...      */
+#define TURBOFNO_ERR_UNSUPPORTED  2  /* transform length outside the built set                           */
+#define TURBOFNO_ERR_WORKSPACE    3  /* workspace missing or too small                                   */
+#define TURBOFNO_ERR_HIP          4  /* the HIP runtime reported a launch error                          */
+
+#define TURBOFNO_MODES 64
+
+/* algorithms of turbofno_layer_2d */
+#define TURBOFNO_2D_AUTO          0
+#define TURBOFNO_2D_THREE_KERNEL  1  /* X transform, fused Y stage, X inverse: the reference's structure */
+#define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM (DX = DY = 256)          */
+
+/*
+ * Fused 1D layer kernel. Replaces the table entries fused_fft_cgemm_ifft[log2(DY)-7]
+ *   fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:15-16 (table), :119-126 (launch)
+ *   fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused_fft_cgemm_ifft_7.cuh:9 (signature
+ *   (int M, int N, int K, float2* FFT_input, float2* B, float2* C, float2* FFT_output, float2 alpha, float2 beta))
+ * M = 64 * S where S = bs*dimX signals per channel. `C` is unused by the reference kernel (its beta*C
+ * term is commented out, fused_fft_cgemm_ifft_7.cuh:186-187) and may be NULL; beta is ignored.
+ * Requires logDY in {7, 8}, M % 64 == 0, N % 64 == 0, K % 8 == 0 (utils/TurboFNO.h:2-4).
+ */
+int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
+                                  float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
+
+/*
+ * X-axis stage kernels of the 2D pipeline. Replace the table entries fft_stride[log2(DX)-7] and
+ * ifft_stride[log2(DX)-7], signature (float2* in, float2* out, int threadblock_bs, int DY, int total, int dimX):
+ *   fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:27-28 (tables), :153-160, :170 (launches)
+ * forward : in[total/DY][DX][DY] -> out[total/DY][dimX][DY]   FFT along DX, first dimX rows kept
+ * backward: in[total/DY][dimX][DY] -> out[total/DY][DX][DY]   rows >= dimX taken as zero, backward FFT along DX
+ * `total` = number of columns (DY * channels * bs). threadblock_bs (columns per block in the
+ * reference) is accepted for signature compatibility and ignored. Requires logDX in {7, 8},
+ * dimX == 64, DY % 16 == 0, total % DY == 0.
+ */
+int turbofno_fft_stride(int logDX, const void* in, void* out, int threadblock_bs, int DY, long total, int dimX,
+                        void* stream);
+int turbofno_ifft_stride(int logDX, const void* in, void* out, int threadblock_bs, int DY, long total, int dimX,
+                         void* stream);
+
+/*
+ * Whole 1D layer, as run by TurboFNO_1D_D for one (bs, dimX, DY, N, K) problem
+ * (fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:104-126). One kernel launch.
+ */
+int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, const void* W, void* y,
+                      float alpha_re, float alpha_im, void* stream);
+
+/*
+ * Whole 2D layer, as run by TurboFNO_2D_D for one (bs, DX, DY, N, K) problem
+ * (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:133-172). The reference keeps its
+ * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
+ * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
+ * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE when DX = DY = 256, else THREE_KERNEL.
+ */
+size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo);
+int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,
+                      float alpha_re, float alpha_im, void* workspace, size_t workspace_bytes, int algo, void* stream);
+
+/* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
+const char* turbofno_last_error_string(void);
+
+/* ABI version of this header (bumped on incompatible change). */
+int turbofno_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TURBOFNO_H */

@@ -1,0 +1,46 @@
+"""CPU-side checks of the boundary: the shared library loads and exports every symbol that
+include/turbofno.h declares; the codelet arithmetic (host build) matches a brute-force DFT."""
+import ctypes
+import os
+import re
+import subprocess
+
+import turbofno_amd as tf
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "turbofno.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(turbofno_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 8
+    L = ctypes.CDLL(tf.library_path())
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_abi_version_and_error_string_without_gpu():
+    L = tf.lib()
+    assert L.turbofno_abi_version() == 1
+    assert L.turbofno_last_error_string() is not None
+    # argument validation happens before any GPU call
+    rc = L.turbofno_fused_fft_cgemm_ifft(8, 64, 64, 12, 1, 1, None, 1, 1.0, 0.0, 0.0, 0.0, None)
+    assert rc == 1 and b"K=12" in L.turbofno_last_error_string()
+    rc = L.turbofno_fused_fft_cgemm_ifft(11, 64, 64, 8, 1, 1, None, 1, 1.0, 0.0, 0.0, 0.0, None)
+    assert rc == 2
+    rc = L.turbofno_layer_2d(1, 256, 256, 8, 64, 1, 1, 1, 1.0, 0.0, None, 0, 0, None)
+    assert rc == 3
+    assert L.turbofno_layer_2d_workspace_bytes(16, 256, 256, 64, 64, 0) == 2 * 64 * 16 * 4096 * 8
+
+
+def test_codelets_on_cpu(tmp_path):
+    exe = str(tmp_path / "codelet_check")
+    subprocess.run(["g++", "-O1", "-std=c++17", os.path.join(ROOT, "tests", "host", "codelet_check.cpp"), "-o", exe],
+                   check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert out.strip().endswith("OK"), out

@@ -1,0 +1,21 @@
+"""turbofno_amd -- MI355X (gfx950) implementation of TurboFNO's fused spectral layer.
+
+The product is libturbofno.so (hand-written HIP kernels behind the C ABI of include/turbofno.h) and
+the C++ drivers under turbofno_amd/host. This module is the thin Python binding used by the tests
+and the benchmark: torch supplies device memory and streams, nothing else. There is no CPU or
+library fallback: if the shared library is missing, importing `turbofno_amd.api` raises.
+"""
+from .api import (  # noqa: F401
+    MODES,
+    TurboFNOError,
+    fft_stride,
+    fused_fft_cgemm_ifft,
+    ifft_stride,
+    layer_1d,
+    layer_2d,
+    layer_2d_workspace_bytes,
+    lib,
+    library_path,
+)
+
+ALGO_AUTO, ALGO_THREE_KERNEL, ALGO_WHOLE_IMAGE = 0, 1, 2

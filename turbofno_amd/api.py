@@ -1,0 +1,129 @@
+"""ctypes binding of libturbofno.so (C ABI: include/turbofno.h).
+
+Function names and argument meaning mirror the reference's kernel tables
+(fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:15-16,
+fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:27-30). Tensors are torch
+complex64 tensors resident on the GPU; every call is asynchronous on torch's current stream.
+"""
+import ctypes
+import os
+
+import torch
+
+MODES = 64
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class TurboFNOError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("turbofno error %d: %s" % (code, message))
+        self.code = code
+
+
+def library_path():
+    return os.path.join(_HERE, "libturbofno.so")
+
+
+def lib():
+    """Loads libturbofno.so; raises (no fallback) when it has not been built."""
+    global _LIB
+    if _LIB is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise ImportError("%s not found: build it with `make -C turbofno_amd/csrc` "
+                              "(or __graft_entry__.build()); there is no fallback path" % path)
+        L = ctypes.CDLL(path)
+        vp, i, l, f, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float, ctypes.c_size_t
+        L.turbofno_fused_fft_cgemm_ifft.argtypes = [i, l, i, i, vp, vp, vp, vp, f, f, f, f, vp]
+        L.turbofno_fft_stride.argtypes = [i, vp, vp, i, i, l, i, vp]
+        L.turbofno_ifft_stride.argtypes = [i, vp, vp, i, i, l, i, vp]
+        L.turbofno_layer_1d.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, vp]
+        L.turbofno_layer_2d_workspace_bytes.argtypes = [i, i, i, i, i, i]
+        L.turbofno_layer_2d_workspace_bytes.restype = sz
+        L.turbofno_layer_2d.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, vp, sz, i, vp]
+        L.turbofno_last_error_string.restype = ctypes.c_char_p
+        L.turbofno_abi_version.restype = i
+        for name in ("turbofno_fused_fft_cgemm_ifft", "turbofno_fft_stride", "turbofno_ifft_stride",
+                     "turbofno_layer_1d", "turbofno_layer_2d"):
+            getattr(L, name).restype = i
+        _LIB = L
+    return _LIB
+
+
+def _check(rc):
+    if rc != 0:
+        raise TurboFNOError(rc, lib().turbofno_last_error_string().decode())
+
+
+def _dev_c64(t, name):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.complex64 and t.is_contiguous()):
+        raise TypeError("%s must be a contiguous complex64 tensor on the GPU" % name)
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _log2(v):
+    return v.bit_length() - 1 if v > 0 and v & (v - 1) == 0 else -1
+
+
+def fused_fft_cgemm_ifft(M, N, K, x, W, y, alpha=1.0 + 0j, beta=0j, C=None):
+    """Fused 1D layer kernel: x[K][S][DY] -> y[N][S][DY], W[k + n*K], M = 64*S (reference signature
+    fused_fft_cgemm_ifft_7.cuh:9; C and beta are unused there and here)."""
+    DY = x.shape[-1]
+    a, b = complex(alpha), complex(beta)
+    _check(lib().turbofno_fused_fft_cgemm_ifft(_log2(DY), M, N, K, _dev_c64(x, "x"), _dev_c64(W, "W"),
+                                               None if C is None else _dev_c64(C, "C"), _dev_c64(y, "y"),
+                                               a.real, a.imag, b.real, b.imag, _stream()))
+    return y
+
+
+def fft_stride(inp, out, threadblock_bs, DY, total, dimX=MODES):
+    """X-axis truncated forward transform: in[total/DY][DX][DY] -> out[total/DY][dimX][DY]."""
+    DX = inp.shape[-2]
+    _check(lib().turbofno_fft_stride(_log2(DX), _dev_c64(inp, "in"), _dev_c64(out, "out"), threadblock_bs, DY,
+                                     total, dimX, _stream()))
+    return out
+
+
+def ifft_stride(inp, out, threadblock_bs, DY, total, dimX=MODES):
+    """X-axis zero-padded backward transform: in[total/DY][dimX][DY] -> out[total/DY][DX][DY]."""
+    DX = out.shape[-2]
+    _check(lib().turbofno_ifft_stride(_log2(DX), _dev_c64(inp, "in"), _dev_c64(out, "out"), threadblock_bs, DY,
+                                      total, dimX, _stream()))
+    return out
+
+
+def layer_1d(x, W, y=None, alpha=1.0 + 0j, dimX=1):
+    """x: [K][bs*dimX][DY], W: [N][K] (element W[k + n*K]) -> y: [N][bs*dimX][DY]."""
+    K, S, DY = x.shape
+    N = W.shape[0]
+    if y is None:
+        y = torch.empty((N, S, DY), dtype=torch.complex64, device=x.device)
+    a = complex(alpha)
+    _check(lib().turbofno_layer_1d(S // dimX, dimX, DY, K, N, _dev_c64(x, "x"), _dev_c64(W, "W"), _dev_c64(y, "y"),
+                                   a.real, a.imag, _stream()))
+    return y
+
+
+def layer_2d_workspace_bytes(bs, DX, DY, K, N, algo=0):
+    return int(lib().turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, algo))
+
+
+def layer_2d(x, W, y=None, alpha=1.0 + 0j, workspace=None, algo=0):
+    """x: [K][bs][DX][DY], W: [N][K] -> y: [N][bs][DX][DY]. `workspace`: uint8 GPU tensor (allocated
+    here when omitted; pass one to keep allocation out of a timed loop)."""
+    K, bs, DX, DY = x.shape
+    N = W.shape[0]
+    if y is None:
+        y = torch.empty((N, bs, DX, DY), dtype=torch.complex64, device=x.device)
+    need = layer_2d_workspace_bytes(bs, DX, DY, K, N, algo)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    a = complex(alpha)
+    _check(lib().turbofno_layer_2d(bs, DX, DY, K, N, _dev_c64(x, "x"), _dev_c64(W, "W"), _dev_c64(y, "y"),
+                                   a.real, a.imag, workspace.data_ptr(), workspace.numel(), algo, _stream()))
+    return y

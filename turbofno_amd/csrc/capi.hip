@@ -1,0 +1,148 @@
+// C ABI of the library: argument validation, dispatch by transform length, error strings.
+// Declarations and the reference interfaces each entry point replaces are in include/turbofno.h.
+#include "../../include/turbofno.h"
+#include "kernels.h"
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_status(hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return TURBOFNO_OK;
+    return fail(TURBOFNO_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int log2_exact(long v)
+{
+    if (v <= 0 || (v & (v - 1))) return -1;
+    int l = 0;
+    while ((1L << l) < v) ++l;
+    return l;
+}
+
+bool length_built(int logD) { return logD == 7 || logD == 8; }
+
+int check_gemm_dims(long M, int N, int K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "M, N, K must be positive (M=%ld N=%d K=%d)", M, N, K);
+    if (M % 64) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld is not a multiple of 64 (64 retained modes per signal)", M);
+    if (N % 64) return fail(TURBOFNO_ERR_INVALID_ARG, "N=%d is not a multiple of the 64-wide output tile", N);
+    if (K % 8) return fail(TURBOFNO_ERR_INVALID_ARG, "K=%d is not a multiple of the 8-deep K tile", K);
+    return TURBOFNO_OK;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int pick_algo(int DX, int DY, int algo) { return algo != TURBOFNO_2D_AUTO ? algo : (DX == 256 && DY == 256 ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL); }
+
+}  // namespace
+
+extern "C" {
+
+int turbofno_abi_version(void) { return 1; }
+
+const char* turbofno_last_error_string(void) { return g_err; }
+
+int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
+                                  float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream)
+{
+    (void)C; (void)beta_re; (void)beta_im;
+    if (!x || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and y must be non-null device pointers");
+    if (int rc = check_gemm_dims(M, N, K)) return rc;
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
+    hipError_t e = tfno::launch_fused_fft_cgemm_ifft(logDY, M / 64, N, K, (const float2*)x, (const float2*)W, (float2*)y,
+                                                     make_float2(alpha_re, alpha_im), (hipStream_t)stream);
+    return hip_status(e, "fused_fft_cgemm_ifft launch");
+}
+
+static int stride_common(bool inverse, int logDX, const void* in, void* out, int DY, long total, int dimX, void* stream)
+{
+    if (!in || !out) return fail(TURBOFNO_ERR_INVALID_ARG, "in and out must be non-null device pointers");
+    if (dimX != TURBOFNO_MODES) return fail(TURBOFNO_ERR_INVALID_ARG, "dimX=%d: exactly 64 rows are retained", dimX);
+    if (DY <= 0 || DY % 16) return fail(TURBOFNO_ERR_INVALID_ARG, "DY=%d must be a positive multiple of 16", DY);
+    if (total <= 0 || total % DY) return fail(TURBOFNO_ERR_INVALID_ARG, "total=%ld must be a positive multiple of DY=%d", total, DY);
+    if (!length_built(logDX)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DX)=%d: only DX in {128, 256} is built", logDX);
+    hipError_t e = inverse ? tfno::launch_ifft_stride(logDX, (const float2*)in, (float2*)out, DY, total / DY, (hipStream_t)stream)
+                           : tfno::launch_fft_stride(logDX, (const float2*)in, (float2*)out, DY, total / DY, (hipStream_t)stream);
+    return hip_status(e, inverse ? "ifft_stride launch" : "fft_stride launch");
+}
+
+int turbofno_fft_stride(int logDX, const void* in, void* out, int threadblock_bs, int DY, long total, int dimX, void* stream)
+{
+    (void)threadblock_bs;
+    return stride_common(false, logDX, in, out, DY, total, dimX, stream);
+}
+
+int turbofno_ifft_stride(int logDX, const void* in, void* out, int threadblock_bs, int DY, long total, int dimX, void* stream)
+{
+    (void)threadblock_bs;
+    return stride_common(true, logDX, in, out, DY, total, dimX, stream);
+}
+
+int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, const void* W, void* y, float alpha_re,
+                      float alpha_im, void* stream)
+{
+    if (bs <= 0 || dimX <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "bs=%d and dimX=%d must be positive", bs, dimX);
+    int logDY = log2_exact(DY);
+    if (logDY < 0) return fail(TURBOFNO_ERR_INVALID_ARG, "DY=%d is not a power of two", DY);
+    return turbofno_fused_fft_cgemm_ifft(logDY, (long)bs * dimX * 64, N, K, x, W, nullptr, y, alpha_re, alpha_im, 0.f, 0.f, stream);
+}
+
+size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo)
+{
+    if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
+    if (pick_algo(DX, DY, algo) == TURBOFNO_2D_WHOLE_IMAGE)
+        return align256((size_t)K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
+    return align256((size_t)K * bs * 64 * DY * sizeof(float2)) + align256((size_t)N * bs * 64 * DY * sizeof(float2));
+}
+
+int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y, float alpha_re,
+                      float alpha_im, void* workspace, size_t workspace_bytes, int algo, void* stream)
+{
+    if (!x || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and y must be non-null device pointers");
+    if (bs <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "bs=%d must be positive", bs);
+    int logDX = log2_exact(DX), logDY = log2_exact(DY);
+    if (logDX < 0 || logDY < 0) return fail(TURBOFNO_ERR_INVALID_ARG, "DX=%d, DY=%d must be powers of two", DX, DY);
+    if (int rc = check_gemm_dims((long)bs * 64 * 64, N, K)) return rc;
+    if (!length_built(logDX) || !length_built(logDY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256} are built", DX, DY);
+    if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE)
+        return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
+    const int a = pick_algo(DX, DY, algo);
+    if (a == TURBOFNO_2D_WHOLE_IMAGE && !(DX == 256 && DY == 256))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "the whole-image algorithm is built for DX = DY = 256 only");
+    const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
+    if (!workspace || workspace_bytes < need)
+        return fail(TURBOFNO_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+    if ((size_t)workspace % 256) return fail(TURBOFNO_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const float2 alpha = make_float2(alpha_re, alpha_im);
+    char* ws = (char*)workspace;
+    if (a == TURBOFNO_2D_WHOLE_IMAGE) {
+        float2* spec = (float2*)ws;
+        float2* cspec = (float2*)(ws + align256((size_t)K * bs * 4096 * sizeof(float2)));
+        if (int rc = hip_status(tfno::launch_fft2d_trunc_256((const float2*)x, spec, (long)K * bs, st), "fft2d_trunc launch")) return rc;
+        if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, st), "cgemm_modes launch")) return rc;
+        return hip_status(tfno::launch_ifft2d_pad_256(cspec, (float2*)y, (long)N * bs, st), "ifft2d_pad launch");
+    }
+    float2* t1 = (float2*)ws;
+    float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));
+    if (int rc = hip_status(tfno::launch_fft_stride(logDX, (const float2*)x, t1, DY, (long)K * bs, st), "fft_stride launch")) return rc;
+    if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, st), "fused_fft_cgemm_ifft launch")) return rc;
+    return hip_status(tfno::launch_ifft_stride(logDX, t2, (float2*)y, DY, (long)N * bs, st), "ifft_stride launch");
+}
+
+}  // extern "C"

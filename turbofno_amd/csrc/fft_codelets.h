@@ -1,0 +1,208 @@
+// Register-resident FFT building blocks for 64-lane wavefronts (gfx950).
+//
+// These replace the reference's auto-generated radix-2 codelets, whose sources live in the empty
+// TurboFFT submodule (include sites: fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/
+// fused_fft_cgemm_ifft_7.cuh:3-4, call sites :46,114,218). A length-D transform (D = 16*L) is split as
+//
+//     y = t + L*i            t < L : lane inside an L-lane group,  i < 16 : register index
+//     G_t[r]   = sum_i v[t + L*i] w16^(i r)                      16-point FFT, all in registers
+//     X[r+16s] = sum_t w_D^(t r) w_L^(t s) G_t[r]                one exchange, then an L-point DFT
+//
+// Truncation to 64 modes means only s < 4 is ever needed ("pruned" second pass: 16 in, 4 out);
+// the zero-padded backward transform is the exact mirror (4 in, 16 out, exchange, 16-point FFT).
+// Discarded and padded modes are therefore never computed, stored or loaded.
+//
+// DIR = -1 is the forward transform exp(-2 pi i jm/D); DIR = +1 the unnormalised backward one.
+#pragma once
+#ifdef TFNO_HOST_CHECK
+// Plain-C++ build of the same arithmetic for the CPU unit test of the codelets (no HIP runtime).
+#include <cmath>
+struct float2 { float x, y; };
+static inline float2 make_float2(float x, float y) { return float2{ x, y }; }
+#define TFNO_DEV static inline
+#define TFNO_TABLE static const
+#else
+#include <hip/hip_runtime.h>
+#define TFNO_DEV __device__ __forceinline__
+#define TFNO_TABLE __device__ __constant__ const
+#endif
+
+namespace tfno {
+
+using cpx = float2;
+
+TFNO_TABLE float2 kTwiddle1024[1024] = {
+#include "twiddles_1024.inc"
+};
+
+TFNO_DEV cpx cadd(cpx a, cpx b) { return make_float2(a.x + b.x, a.y + b.y); }
+TFNO_DEV cpx csub(cpx a, cpx b) { return make_float2(a.x - b.x, a.y - b.y); }
+TFNO_DEV cpx cmul(cpx a, cpx b) { return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x); }
+TFNO_DEV cpx cmulc(cpx a, cpx b) { return make_float2(a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y); }  // a * conj(b)
+TFNO_DEV void cfma(cpx& acc, cpx a, cpx b)
+{
+    acc.x = fmaf(a.x, b.x, acc.x); acc.x = fmaf(-a.y, b.y, acc.x);
+    acc.y = fmaf(a.x, b.y, acc.y); acc.y = fmaf(a.y, b.x, acc.y);
+}
+
+// multiply by DIR * i   (forward: -i, backward: +i)
+template <int DIR> TFNO_DEV cpx mul_dir_i(cpx a)
+{
+    return DIR < 0 ? make_float2(a.y, -a.x) : make_float2(-a.y, a.x);
+}
+
+// w16^k for the forward direction, k = 0..15 (compile-time constants)
+template <int K16> TFNO_DEV constexpr float w16_re()
+{
+    constexpr float c[16] = { 1.0f, 0.92387953251128674f, 0.70710678118654752f, 0.38268343236508977f,
+                              0.0f, -0.38268343236508977f, -0.70710678118654752f, -0.92387953251128674f,
+                              -1.0f, -0.92387953251128674f, -0.70710678118654752f, -0.38268343236508977f,
+                              0.0f, 0.38268343236508977f, 0.70710678118654752f, 0.92387953251128674f };
+    return c[K16 & 15];
+}
+template <int K16> TFNO_DEV constexpr float w16_im()
+{
+    constexpr float s[16] = { 0.0f, -0.38268343236508977f, -0.70710678118654752f, -0.92387953251128674f,
+                              -1.0f, -0.92387953251128674f, -0.70710678118654752f, -0.38268343236508977f,
+                              0.0f, 0.38268343236508977f, 0.70710678118654752f, 0.92387953251128674f,
+                              1.0f, 0.92387953251128674f, 0.70710678118654752f, 0.38268343236508977f };
+    return s[K16 & 15];
+}
+
+// a * w16^(DIR-signed k)
+template <int DIR, int K16> TFNO_DEV cpx mul_w16(cpx a)
+{
+    constexpr int k = K16 & 15;
+    if constexpr (k == 0) return a;
+    else if constexpr (k == 4) return mul_dir_i<DIR>(a);
+    else if constexpr (k == 8) return make_float2(-a.x, -a.y);
+    else if constexpr (k == 12) return mul_dir_i<-DIR>(a);
+    else {
+        constexpr float wr = w16_re<k>();
+        constexpr float wi = DIR < 0 ? w16_im<k>() : -w16_im<k>();
+        return make_float2(a.x * wr - a.y * wi, a.x * wi + a.y * wr);
+    }
+}
+
+// 4-point butterfly, in place, natural order out
+template <int DIR> TFNO_DEV void radix4(cpx& a0, cpx& a1, cpx& a2, cpx& a3)
+{
+    cpx t0 = cadd(a0, a2), t1 = csub(a0, a2), t2 = cadd(a1, a3), t3 = mul_dir_i<DIR>(csub(a1, a3));
+    a0 = cadd(t0, t2); a1 = cadd(t1, t3); a2 = csub(t0, t2); a3 = csub(t1, t3);
+}
+
+// position of output bin r inside the array after fft16(): X[r] = v[fft16_slot(r)]
+TFNO_DEV constexpr int fft16_slot(int r) { return (r >> 2) | ((r & 3) << 2); }
+
+// 16-point FFT in registers. Input natural order v[i]; output bin r is left in v[fft16_slot(r)].
+template <int DIR> TFNO_DEV void fft16(cpx (&v)[16])
+{
+#pragma unroll
+    for (int i0 = 0; i0 < 4; ++i0) radix4<DIR>(v[i0], v[i0 + 4], v[i0 + 8], v[i0 + 12]);
+    // v[i0 + 4 rho] = B[i0][rho]; twiddle by w16^(i0*rho)
+    v[5] = mul_w16<DIR, 1>(v[5]);   v[9] = mul_w16<DIR, 2>(v[9]);   v[13] = mul_w16<DIR, 3>(v[13]);
+    v[6] = mul_w16<DIR, 2>(v[6]);   v[10] = mul_w16<DIR, 4>(v[10]); v[14] = mul_w16<DIR, 6>(v[14]);
+    v[7] = mul_w16<DIR, 3>(v[7]);   v[11] = mul_w16<DIR, 6>(v[11]); v[15] = mul_w16<DIR, 9>(v[15]);
+#pragma unroll
+    for (int rho = 0; rho < 4; ++rho) radix4<DIR>(v[4 * rho], v[4 * rho + 1], v[4 * rho + 2], v[4 * rho + 3]);
+}
+
+// First four bins (s = 0..3) of a 16-point DFT of g[0..15]:  out[s] = sum_t g[t] w16^(t s).
+template <int DIR> TFNO_DEV void dft16_first4(cpx (&g)[16], cpx (&out)[4])
+{
+#pragma unroll
+    for (int t0 = 0; t0 < 4; ++t0) radix4<DIR>(g[t0], g[t0 + 4], g[t0 + 8], g[t0 + 12]);
+    // g[t0 + 4 s] = sum_t1 g[t0 + 4 t1] w4^(t1 s);  out[s] = sum_t0 w16^(t0 s) g[t0 + 4 s]
+    out[0] = cadd(cadd(g[0], g[1]), cadd(g[2], g[3]));
+    out[1] = cadd(cadd(g[4], mul_w16<DIR, 1>(g[5])), cadd(mul_w16<DIR, 2>(g[6]), mul_w16<DIR, 3>(g[7])));
+    out[2] = cadd(cadd(g[8], mul_w16<DIR, 2>(g[9])), cadd(mul_w16<DIR, 4>(g[10]), mul_w16<DIR, 6>(g[11])));
+    out[3] = cadd(cadd(g[12], mul_w16<DIR, 3>(g[13])), cadd(mul_w16<DIR, 6>(g[14]), mul_w16<DIR, 9>(g[15])));
+}
+
+// 16-point DFT of a 4-element input padded with 12 zeros:  h[t] = sum_{s<4} c[s] w16^(t s), t = 0..15.
+template <int DIR> TFNO_DEV void dft16_pad4(const cpx (&c)[4], cpx (&h)[16])
+{
+    // t = t0 + 4 t1:  h[t0 + 4 t1] = sum_s (c[s] w16^(t0 s)) w4^(t1 s)
+    {
+        cpx d0 = c[0], d1 = c[1], d2 = c[2], d3 = c[3];
+        radix4<DIR>(d0, d1, d2, d3); h[0] = d0; h[4] = d1; h[8] = d2; h[12] = d3;
+    }
+    {
+        cpx d0 = c[0], d1 = mul_w16<DIR, 1>(c[1]), d2 = mul_w16<DIR, 2>(c[2]), d3 = mul_w16<DIR, 3>(c[3]);
+        radix4<DIR>(d0, d1, d2, d3); h[1] = d0; h[5] = d1; h[9] = d2; h[13] = d3;
+    }
+    {
+        cpx d0 = c[0], d1 = mul_w16<DIR, 2>(c[1]), d2 = mul_w16<DIR, 4>(c[2]), d3 = mul_w16<DIR, 6>(c[3]);
+        radix4<DIR>(d0, d1, d2, d3); h[2] = d0; h[6] = d1; h[10] = d2; h[14] = d3;
+    }
+    {
+        cpx d0 = c[0], d1 = mul_w16<DIR, 3>(c[1]), d2 = mul_w16<DIR, 6>(c[2]), d3 = mul_w16<DIR, 9>(c[3]);
+        radix4<DIR>(d0, d1, d2, d3); h[3] = d0; h[7] = d1; h[11] = d2; h[15] = d3;
+    }
+}
+
+// First four bins of an 8-point DFT:  out[s] = sum_{t<8} g[t] w8^(t s), s = 0..3.
+template <int DIR> TFNO_DEV void dft8_first4(cpx (&g)[8], cpx (&out)[4])
+{
+    // t = t0 + 2 t1:  B[t0][s] = sum_t1 g[t0 + 2 t1] w4^(t1 s);  out[s] = B[0][s] + w8^s B[1][s]
+    radix4<DIR>(g[0], g[2], g[4], g[6]);
+    radix4<DIR>(g[1], g[3], g[5], g[7]);
+    out[0] = cadd(g[0], g[1]);
+    out[1] = cadd(g[2], mul_w16<DIR, 2>(g[3]));
+    out[2] = cadd(g[4], mul_w16<DIR, 4>(g[5]));
+    out[3] = cadd(g[6], mul_w16<DIR, 6>(g[7]));
+}
+
+// 8-point DFT of a 4-element input padded with 4 zeros:  h[t] = sum_{s<4} c[s] w8^(t s), t = 0..7.
+template <int DIR> TFNO_DEV void dft8_pad4(const cpx (&c)[4], cpx (&h)[8])
+{
+    {
+        cpx d0 = c[0], d1 = c[1], d2 = c[2], d3 = c[3];
+        radix4<DIR>(d0, d1, d2, d3); h[0] = d0; h[2] = d1; h[4] = d2; h[6] = d3;
+    }
+    {
+        cpx d0 = c[0], d1 = mul_w16<DIR, 2>(c[1]), d2 = mul_w16<DIR, 4>(c[2]), d3 = mul_w16<DIR, 6>(c[3]);
+        radix4<DIR>(d0, d1, d2, d3); h[1] = d0; h[3] = d1; h[5] = d2; h[7] = d3;
+    }
+}
+
+// Per-lane inter-pass twiddles  tw[r] = w_D^(t r), r = 0..15, for lane t of an L-lane group (D = 16 L).
+template <int LOGD> TFNO_DEV void load_lane_twiddles(int t, cpx (&tw)[16])
+{
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tw[r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
+}
+
+// Forward first pass: 16-point FFT of the lane's strided samples, then the inter-pass twiddle.
+// On return g[r] (natural order) = w_D^(t r) * G_t[r].
+TFNO_DEV void fwd_pass1(cpx (&v)[16], const cpx (&tw)[16], cpx (&g)[16])
+{
+    fft16<-1>(v);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) g[r] = (r == 0) ? v[0] : cmul(v[fft16_slot(r)], tw[r]);
+}
+
+// Backward last pass: conj twiddle, 16-point backward FFT. e[r] in natural order; on return
+// y[i] = value of output sample t + L*i.
+TFNO_DEV void inv_pass2(cpx (&e)[16], const cpx (&tw)[16], cpx (&y)[16])
+{
+#pragma unroll
+    for (int r = 1; r < 16; ++r) e[r] = cmulc(e[r], tw[r]);
+    fft16<+1>(e);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = e[fft16_slot(i)];
+}
+
+// Orders LDS traffic of one wavefront: everything the wave wrote before is visible to its own
+// lanes after. DS operations of a wave complete in issue order, so no hardware wait is needed
+// beyond what the compiler inserts for the data dependency; this only stops compiler reordering.
+#ifndef TFNO_HOST_CHECK
+TFNO_DEV void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+#endif
+
+}  // namespace tfno

@@ -1,0 +1,75 @@
+// Transforms of one signal by one L-lane group of a wavefront (L = D/16 lanes, 16 samples per lane),
+// built from the register codelets plus one padded LDS exchange that stays inside the wavefront
+// (no block barrier). Shared by the fused 1D kernel and the 2D image kernels.
+#pragma once
+#include "fft_codelets.h"
+
+namespace tfno {
+
+template <int LOGDY> struct Geo1D {
+    static constexpr int DY = 1 << LOGDY;
+    static constexpr int L = DY / 16;        // lanes per signal
+    static constexpr int GROUPS = 256 / L;   // signals transformed concurrently = K chunk
+    static constexpr int MM = 64 / L;        // modes owned per lane   (m = lane + L*mm)
+    static constexpr int NN = 64 / GROUPS;   // output channels per group (n = g + GROUPS*jn)
+    static constexpr int EXCH = L * 17;      // complex per group exchange region
+    static constexpr int SA_PITCH = 64;
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * 64 + GROUPS * EXCH);
+};
+
+// forward transform of one signal by one L-lane group; lane t holds samples t + L*i in v[].
+// On return lane `t` holds modes m = t + L*mm in out[mm].
+template <int LOGDY>
+TFNO_DEV void group_forward(cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
+{
+    constexpr int L = Geo1D<LOGDY>::L;
+    cpx g[16];
+    fwd_pass1(v, tw, g);
+    wave_lds_fence();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) exch[t * 17 + r] = g[r];
+    wave_lds_fence();
+    if constexpr (L == 16) {
+        cpx u[16];
+#pragma unroll
+        for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
+        dft16_first4<-1>(u, out);                       // out[s] = X[t + 16 s]
+    } else {
+        cpx u0[8], u1[8], o0[4], o1[4];
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) { u0[tt] = exch[tt * 17 + t]; u1[tt] = exch[tt * 17 + t + 8]; }
+        dft8_first4<-1>(u0, o0);                        // X[t + 16 s]
+        dft8_first4<-1>(u1, o1);                        // X[t + 8 + 16 s]
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { out[2 * s] = o0[s]; out[2 * s + 1] = o1[s]; }
+    }
+}
+
+// zero-padded backward transform; lane t holds modes m = t + L*mm in c[]; returns samples t + L*i in y[].
+template <int LOGDY>
+TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[16], cpx* exch, int t, cpx (&y)[16])
+{
+    constexpr int L = Geo1D<LOGDY>::L;
+    wave_lds_fence();
+    if constexpr (L == 16) {
+        cpx h[16];
+        dft16_pad4<+1>(c, h);
+#pragma unroll
+        for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+    } else {
+        cpx c0[4], c1[4], h0[8], h1[8];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { c0[s] = c[2 * s]; c1[s] = c[2 * s + 1]; }
+        dft8_pad4<+1>(c0, h0);
+        dft8_pad4<+1>(c1, h1);
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) { exch[tt * 17 + t] = h0[tt]; exch[tt * 17 + t + 8] = h1[tt]; }
+    }
+    wave_lds_fence();
+    cpx e[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+    inv_pass2(e, tw, y);
+}
+
+}  // namespace tfno

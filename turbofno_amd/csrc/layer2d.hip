@@ -1,0 +1,215 @@
+// Whole-image 2D spectral layer for 256 x 256 grids (the MI355X-first path of the 2D layer).
+//
+// The reference's "fully fused" 2D variant is three kernels with two HBM round trips of
+// half-truncated intermediates (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:150-172:
+// X transform -> t1[K*bs][64][DY], fused Y stage, t2[N*bs][64][DY] -> X inverse). Here one 1024-thread
+// block owns a whole 256 x 256 image, so only fully truncated 64 x 64 spectra (1/16 of the image)
+// ever leave the CU:
+//
+//   fft2d_trunc_256   image (k,b): 256 row FFTs along Y (coalesced 2 KiB rows, 64 modes kept, held in
+//                     registers), redistribution through LDS, 64 column FFTs along X (64 modes kept)
+//                     -> spec[k][b][4096]                                       reads 512 KiB, writes 32 KiB
+//   cgemm_modes       C[n][b][m] = alpha * sum_k W[k][n] spec[k][b][m] on the fp32 matrix cores
+//   ifft2d_pad_256    exact mirror -> y[n][b][256][256]                         reads 32 KiB, writes 512 KiB
+//
+// so x is read once and y written once; padded / discarded modes are never touched in memory.
+// The 4096 modes of an image are stored in "lane order": element s*1024 + q*16 + r holds mode
+// (p = r + 16 s, q). That order is private to these three kernels (producer and consumer lanes
+// coincide, every access is a contiguous 512 B per wavefront) and the GEMM is oblivious to it.
+#include "group_fft.h"
+#include "kernels.h"
+
+namespace tfno {
+
+namespace {
+constexpr int IMG = 256;
+constexpr int TPITCH = 66;                       // row pitch (complex) of the 256 x 64 redistribution tile
+constexpr int EXCH256 = 16 * 17;                 // exchange region of one 16-lane group
+constexpr size_t LDS2D_BYTES = sizeof(float2) * (size_t)(64 * EXCH256 > IMG * TPITCH ? 64 * EXCH256 : IMG * TPITCH);
+
+// Row handled by 16-lane group j of wave w in pass `it`: groups 0/1 of a wave are 8 rows apart so the
+// two groups that share an LDS cycle hit disjoint banks in the pitch-66 tile.
+__device__ __forceinline__ int row_of(int w, int j, int it)
+{
+    return 64 * it + ((w & 7) | ((j & 1) << 3) | ((j >> 1) << 4) | ((w >> 3) << 5));
+}
+}  // namespace
+
+__global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec)
+{
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
+    const long img = blockIdx.x;
+    float2* exch = lds + g * EXCH256;
+
+    cpx tw[16];
+    load_lane_twiddles<8>(r, tw);
+
+    // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row_of(w, j, it)
+    cpx T[4][4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const float2* src = x + (img * IMG + row_of(w, j, it)) * IMG + r;
+        cpx v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = src[16 * i];
+        group_forward<8>(v, tw, exch, r, T[it]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) lds[row_of(w, j, it) * TPITCH + r + 16 * s] = T[it][s];
+    __syncthreads();
+    // pass 2: columns (along X); group g owns column q = g, lane r holds rows r + 16 i
+    cpx v[16], z[4];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = lds[(r + 16 * i) * TPITCH + g];
+    __syncthreads();
+    group_forward<8>(v, tw, exch, r, z);
+    float2* dst = spec + img * 4096 + tid;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) dst[1024 * s] = z[s];
+}
+
+__global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __restrict__ spec, float2* __restrict__ y)
+{
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
+    const long img = blockIdx.x;
+    float2* exch = lds + g * EXCH256;
+
+    cpx tw[16];
+    load_lane_twiddles<8>(r, tw);
+
+    // pass 1: columns (p -> x) of column q = g
+    {
+        const float2* src = spec + img * 4096 + tid;
+        cpx c[4], u[16];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) c[s] = src[1024 * s];
+        group_backward<8>(c, tw, exch, r, u);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) lds[(r + 16 * i) * TPITCH + g] = u[i];
+    }
+    __syncthreads();
+    cpx cc[4][4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) cc[it][s] = lds[row_of(w, j, it) * TPITCH + r + 16 * s];
+    __syncthreads();
+    // pass 2: rows (q -> y), coalesced 2 KiB row stores
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        cpx yv[16];
+        group_backward<8>(cc[it], tw, exch, r, yv);
+        float2* dst = y + (img * IMG + row_of(w, j, it)) * IMG + r;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[16 * i] = yv[i];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Mode-space complex GEMM on the fp32 matrix cores.
+//   C[n][m] = alpha * sum_k W[k + n*K] * A[k][m],   A: [K][Mtot], C: [N][Mtot]  (m contiguous)
+// Same contraction as the reference's cgemm / the GEMM phase of its fused kernel
+// (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4-205, operand layout lda=M, ldb=K, ldc=M),
+// expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition) on
+// v_mfma_f32_32x32x2_f32: rows = (n, re/im), cols = 32 consecutive m, contraction = (k, re/im).
+// One wave owns a 32-m strip and a 64-channel n tile (4 accumulators of 32x32).
+// ---------------------------------------------------------------------------------------------
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int GEMM_KC = 64;      // channels per LDS-resident W chunk
+
+__global__ __launch_bounds__(256) void cgemm_modes_kernel(const float2* __restrict__ A, const float2* __restrict__ W,
+                                                          float2* __restrict__ C, long Mtot, int N, int K, float2 alpha)
+{
+    // sW[(k*128 + n')*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:  {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1
+    __shared__ float sW[GEMM_KC * 128 * 2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
+    const long m0 = ((long)blockIdx.x * 4 + wave) * 32;
+    const int n0 = blockIdx.y * 64;
+
+    floatx16 acc[4];
+#pragma unroll
+    for (int tI = 0; tI < 4; ++tI)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[tI][e] = 0.f;
+
+    for (int kc = 0; kc < K; kc += GEMM_KC) {
+        const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;
+        __syncthreads();
+        for (int idx = tid; idx < GEMM_KC * 64; idx += 256) {
+            int n = idx % 64, k = idx / 64;   // n fastest: conflict-free 16 B LDS stores
+            float2 w = make_float2(0.f, 0.f);
+            if (k < kn) {
+                float2 w0 = W[(kc + k) + (long)(n0 + n) * K];
+                w = make_float2(w0.x * alpha.x - w0.y * alpha.y, w0.x * alpha.y + w0.y * alpha.x);
+            }
+            *reinterpret_cast<float4*>(&sW[(k * 128 + 2 * n) * 2]) = make_float4(w.x, -w.y, w.y, w.x);
+        }
+        __syncthreads();
+        // lane (col, half) feeds A[kc + kk + half][m0 + col] as {re, im}: two contraction steps
+        const float2* ap = A + (long)(kc + half) * Mtot + m0 + col;
+#pragma unroll 4
+        for (int kk = 0; kk < kn; kk += 2) {
+            float2 b = ap[(long)kk * Mtot];
+#pragma unroll
+            for (int tI = 0; tI < 4; ++tI) {
+                float2 a = *reinterpret_cast<const float2*>(&sW[((kk + half) * 128 + tI * 32 + col) * 2]);
+                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc[tI], 0, 0, 0);
+                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc[tI], 0, 0, 0);
+            }
+        }
+    }
+    // D[row = 8 i + 4 half + jj*2 + c'][col]: row = 2 n_local + c'
+#pragma unroll
+    for (int tI = 0; tI < 4; ++tI)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                int n = n0 + tI * 16 + 4 * i + 2 * half + jj;
+                C[(long)n * Mtot + m0 + col] = make_float2(acc[tI][4 * i + 2 * jj], acc[tI][4 * i + 2 * jj + 1]);
+            }
+}
+
+hipError_t launch_fft2d_trunc_256(const float2* x, float2* spec, long nimg, hipStream_t stream)
+{
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fft2d_trunc_256_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)nimg), dim3(1024), LDS2D_BYTES, stream, x, spec);
+    return hipGetLastError();
+}
+
+hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipStream_t stream)
+{
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ifft2d_pad_256_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(ifft2d_pad_256_kernel, dim3((unsigned)nimg), dim3(1024), LDS2D_BYTES, stream, spec, y);
+    return hipGetLastError();
+}
+
+hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
+                              hipStream_t stream)
+{
+    if (Mtot % 128 != 0 || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(Mtot / 128), (unsigned)(N / 64), 1);
+    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(256), 0, stream, A, W, C, Mtot, N, K, alpha);
+    return hipGetLastError();
+}
+
+}  // namespace tfno

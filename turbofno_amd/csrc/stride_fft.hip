@@ -1,0 +1,147 @@
+// X-axis transforms of the three-kernel 2D pipeline: forward FFT along DX (element stride DY) with
+// truncation to the first 64 rows, and its mirror, zero-padding 64 rows to DX and transforming back.
+//
+// Replace fft_N_stride / ifft_N_stride of the reference's missing TurboFFT submodule, launched at
+// fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:153-160 and :170:
+//   forward   in[sig][DX][DY]  -> out[sig][64][DY]
+//   backward  in[sig][64][DY]  -> out[sig][DX][DY]
+// A block owns 16 adjacent columns (128 contiguous bytes per row, one full cache line; the reference
+// uses 4 columns = 32 bytes) and all DX rows; thread (yl, t) holds rows t + L*i of column yl in
+// registers, runs the 16-point pass there, and the single exchange goes through LDS laid out
+// [t][r][yl] so that both the writes and the reads are conflict free on 64 banks.
+#include "fft_codelets.h"
+#include "kernels.h"
+
+namespace tfno {
+
+template <int LOGDX> struct GeoStride {
+    static constexpr int DX = 1 << LOGDX;
+    static constexpr int L = DX / 16;
+    static constexpr int THREADS = 16 * L;
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(L * 17 * 16);
+};
+
+template <int LOGDX>
+__global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void fft_stride_kernel(const float2* __restrict__ in,
+                                                                              float2* __restrict__ out, int DY)
+{
+    using G = GeoStride<LOGDX>;
+    constexpr int DX = G::DX, L = G::L;
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, yl = tid & 15, t = tid >> 4;
+    const long col = (long)blockIdx.x * 16 + yl;
+    const long sig = col / DY;
+    const int y = (int)(col % DY);
+
+    cpx tw[16], v[16], g[16];
+    load_lane_twiddles<LOGDX>(t, tw);
+    const float2* src = in + (sig * DX + t) * DY + y;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = src[(long)L * i * DY];
+    fwd_pass1(v, tw, g);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lds[(t * 17 + r) * 16 + yl] = g[r];
+    __syncthreads();
+    float2* dst = out + sig * 64 * DY + y;
+    if constexpr (L == 16) {
+        cpx u[16], o[4];
+#pragma unroll
+        for (int tt = 0; tt < 16; ++tt) u[tt] = lds[(tt * 17 + t) * 16 + yl];
+        dft16_first4<-1>(u, o);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) dst[(long)(t + 16 * s) * DY] = o[s];
+    } else {
+        cpx u0[8], u1[8], o0[4], o1[4];
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) {
+            u0[tt] = lds[(tt * 17 + t) * 16 + yl];
+            u1[tt] = lds[(tt * 17 + t + 8) * 16 + yl];
+        }
+        dft8_first4<-1>(u0, o0);
+        dft8_first4<-1>(u1, o1);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            dst[(long)(t + 16 * s) * DY] = o0[s];
+            dst[(long)(t + 8 + 16 * s) * DY] = o1[s];
+        }
+    }
+}
+
+template <int LOGDX>
+__global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void ifft_stride_kernel(const float2* __restrict__ in,
+                                                                               float2* __restrict__ out, int DY)
+{
+    using G = GeoStride<LOGDX>;
+    constexpr int DX = G::DX, L = G::L;
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, yl = tid & 15, t = tid >> 4;
+    const long col = (long)blockIdx.x * 16 + yl;
+    const long sig = col / DY;
+    const int y = (int)(col % DY);
+
+    cpx tw[16];
+    load_lane_twiddles<LOGDX>(t, tw);
+    const float2* src = in + sig * 64 * DY + y;
+    if constexpr (L == 16) {
+        cpx c[4], h[16];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) c[s] = src[(long)(t + 16 * s) * DY];
+        dft16_pad4<+1>(c, h);
+#pragma unroll
+        for (int tt = 0; tt < 16; ++tt) lds[(tt * 17 + t) * 16 + yl] = h[tt];
+    } else {
+        cpx c0[4], c1[4], h0[8], h1[8];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            c0[s] = src[(long)(t + 16 * s) * DY];
+            c1[s] = src[(long)(t + 8 + 16 * s) * DY];
+        }
+        dft8_pad4<+1>(c0, h0);
+        dft8_pad4<+1>(c1, h1);
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) {
+            lds[(tt * 17 + t) * 16 + yl] = h0[tt];
+            lds[(tt * 17 + t + 8) * 16 + yl] = h1[tt];
+        }
+    }
+    __syncthreads();
+    cpx e[16], yv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * 16 + yl];
+    inv_pass2(e, tw, yv);
+    float2* dst = out + (sig * DX + t) * DY + y;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dst[(long)L * i * DY] = yv[i];
+}
+
+template <int LOGDX, bool INVERSE>
+static hipError_t launch_stride_t(const float2* in, float2* out, int DY, long nsig, hipStream_t stream)
+{
+    using G = GeoStride<LOGDX>;
+    long blocks = nsig * DY / 16;
+    if (blocks <= 0 || blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)blocks, 1, 1), block(G::THREADS, 1, 1);
+    if (INVERSE) hipLaunchKernelGGL(ifft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
+    else hipLaunchKernelGGL(fft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
+    return hipGetLastError();
+}
+
+hipError_t launch_fft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream)
+{
+    switch (logDX) {
+    case 7: return launch_stride_t<7, false>(in, out, DY, nsig, stream);
+    case 8: return launch_stride_t<8, false>(in, out, DY, nsig, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream)
+{
+    switch (logDX) {
+    case 7: return launch_stride_t<7, true>(in, out, DY, nsig, stream);
+    case 8: return launch_stride_t<8, true>(in, out, DY, nsig, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace tfno
