@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused spectral layer on one MI355X.
+
+One "step" = one pass of the 2D layer (FFT2 -> keep 64x64 modes -> CGEMM over channels -> pad ->
+iFFT2) over the headline batch: bs=16, 256x256 grid, K=N=64, complex64, inputs resident in HBM.
+Prints ONE JSON line (see the keys below). The timed region contains only library calls through
+the C ABI; the CPU oracle is used solely for the separately reported cpu_baseline leg.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--bs", type=int, default=16)
+    ap.add_argument("--algo", type=int, default=0, help="0 auto, 1 three-kernel pipeline, 2 whole-image")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-comparators", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build targets ONE GPU (the layer shards over the batch with no exchange; "
+              "multi-GPU runs are not part of it). Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import turbofno_amd as tf
+    from turbofno_amd import workloads
+
+    bs, DX, DY, K, N = args.bs, 256, 256, 64, 64
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    x_h, W_h = workloads.vorticity_2d(0x5EED + 5, bs, DX, DY, K, N)
+    x = torch.from_numpy(x_h).to(dev)
+    W = torch.from_numpy(W_h).to(dev)
+    y = torch.empty((N, bs, DX, DY), dtype=torch.complex64, device=dev)
+    ws = torch.empty(tf.layer_2d_workspace_bytes(bs, DX, DY, K, N, args.algo), dtype=torch.uint8, device=dev)
+
+    def step():
+        tf.layer_2d(x, W, y=y, alpha=1.0, workspace=ws, algo=args.algo)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = e0.elapsed_time(e1) / args.steps
+
+    img_bytes = 8 * bs * DX * DY
+    layer_bytes = img_bytes * (K + N) + 8 * K * N
+
+    # ---- per-stage timing of the same steps (HIP events on the launch stream) ----------------------
+    roofline = None
+    stages = {}
+    algo = args.algo if args.algo else 2
+    if algo == 2:
+        spec = torch.empty((K * bs, 4096), dtype=torch.complex64, device=dev)
+        cspec = torch.empty((N * bs, 4096), dtype=torch.complex64, device=dev)
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        for s in range(args.steps):
+            ev[s][0].record(); tf.fft2d_trunc(x, spec)
+            ev[s][1].record(); tf.cgemm(bs * 4096, N, K, spec, W, cspec, 1.0)
+            ev[s][2].record(); tf.ifft2d_pad(cspec, y)
+            ev[s][3].record()
+        torch.cuda.synchronize()
+        names = ["fft2d_trunc_256", "cgemm_modes", "ifft2d_pad_256"]
+        for i, nme in enumerate(names):
+            stages[nme] = float(np.mean([ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(args.steps)]))
+        # dominant kernel = the longer of the two image kernels; its algorithmic bytes = one pass over
+        # its side of the layer (input read once / output written once)
+        dom = max(("fft2d_trunc_256", "ifft2d_pad_256"), key=lambda k: stages[k])
+        dom_bytes = img_bytes * (K if dom == "fft2d_trunc_256" else N)
+        achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "algorithmic_bytes_per_launch": dom_bytes}
+    else:
+        achieved = layer_bytes / (ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "three-kernel pipeline (whole layer)", "achieved": round(achieved, 1),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "algorithmic_bytes_per_launch": layer_bytes}
+
+    layer_gbs = layer_bytes / (ms * 1e-3) / 1e9
+
+    # ---- comparators on the same inputs (informational) ------------------------------------------
+    comparators = {}
+    if not args.no_comparators:
+        def timed(fn, reps):
+            fn(); torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record(); torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps
+        if algo == 2:
+            ws3 = torch.empty(tf.layer_2d_workspace_bytes(bs, DX, DY, K, N, 1), dtype=torch.uint8, device=dev)
+            comparators["three_kernel_pipeline_ms"] = round(
+                timed(lambda: tf.layer_2d(x, W, y=y, alpha=1.0, workspace=ws3, algo=1), 5), 4)
+            del ws3
+
+        def unfused_library():
+            # unfused sequence through vendor libraries (rocFFT + rocBLAS via torch): FFT2, truncate, GEMM, pad, iFFT2
+            A = torch.fft.fft2(x)[..., :64, :64]
+            C = torch.einsum("kbpq,nk->nbpq", A, W)
+            Cp = torch.zeros((N, bs, DX, DY), dtype=torch.complex64, device=dev)
+            Cp[..., :64, :64] = C
+            return torch.fft.ifft2(Cp, norm="forward")
+        try:
+            comparators["unfused_rocfft_rocblas_ms"] = round(timed(unfused_library, 3), 4)
+        except Exception as exc:  # pragma: no cover - informational only
+            comparators["unfused_rocfft_rocblas_ms"] = "failed: %s" % type(exc).__name__
+
+    # ---- CPU baseline: fp32 OpenMP restatement of the library baseline, bounded sample -------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        sample_bs = 2
+        xs = np.ascontiguousarray(x_h[:, :sample_bs])
+        cores = min(oracle.cpu_threads(), os.cpu_count() or 1)
+        best = 1e30
+        reps = 0
+        t_start = time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t_start < 10.0 and reps < 20):
+            t = time.perf_counter()
+            oracle.cpu_baseline_layer_2d(xs, W_h, 1.0, cores)
+            best = min(best, time.perf_counter() - t)
+            reps += 1
+        cpu = {"value": round(best * 1e3 * (bs / sample_bs), 2), "unit": "ms/layer", "cores": cores, "kind": "port",
+               "sample": "bs=%d of the same workload (K=N=64, 256x256), best of %d runs, scaled x%d to bs=%d"
+                         % (sample_bs, reps, bs // sample_bs, bs)}
+
+    out = {
+        "metric": "fused FFT-CGEMM-iFFT ms/layer, 2D bs=%d 256x256 K=N=64" % bs,
+        "value": round(ms, 4), "unit": "ms/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "complex64 (fp32 arithmetic)", "data": "synthetic",
+        "config": {"workload": "2D layer bs=%d 256x256 K=64 N=64, 64x64 modes, Gaussian random field input" % bs,
+                   "algo": {0: "auto(whole-image)", 1: "three-kernel", 2: "whole-image"}[args.algo]},
+        "layer_algorithmic_bytes": layer_bytes, "layer_GBps": round(layer_gbs, 1),
+        "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall_ms, 4),
+        "stage_ms": {k: round(v, 4) for k, v in stages.items()},
+        "roofline": roofline, "cpu_baseline": cpu, "comparators": comparators,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -86,6 +86,25 @@ size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, i
 int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,
                       float alpha_re, float alpha_im, void* workspace, size_t workspace_bytes, int algo, void* stream);
 
+/*
+ * Stages of the whole-image 2D algorithm, exposed so that they can be timed, profiled and composed
+ * individually (the reference's variants A/B/C compose the same layer from separately launched stages).
+ *   turbofno_fft2d_trunc : x[nimg][DX][DY] -> spec[nimg][4096]  truncated 2D forward transform per image
+ *   turbofno_ifft2d_pad  : spec[nimg][4096] -> y[nimg][DX][DY]  zero-padded 2D backward transform per image
+ * The 4096 retained modes of an image are stored in an order private to these two kernels (element
+ * s*1024 + q*16 + r holds mode (p = r + 16 s, q)); a GEMM over the channel dimension does not care.
+ * Requires DX = DY = 256.
+ *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] (column major, lda = M, ldb = K,
+ *   ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
+ *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:182-200) for beta = 0,
+ *   the only value with which the fused variant D uses the product. Requires M % 128 == 0, N % 64 == 0,
+ *   K % 8 == 0.
+ */
+int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream);
+int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, void* stream);
+int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im,
+                   void* stream);
+
 /* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
 const char* turbofno_last_error_string(void);
 

@@ -8,6 +8,9 @@ library fallback: if the shared library is missing, importing `turbofno_amd.api`
 from .api import (  # noqa: F401
     MODES,
     TurboFNOError,
+    cgemm,
+    fft2d_trunc,
+    ifft2d_pad,
     fft_stride,
     fused_fft_cgemm_ifft,
     ifft_stride,

@@ -42,10 +42,14 @@ def lib():
         L.turbofno_layer_2d_workspace_bytes.argtypes = [i, i, i, i, i, i]
         L.turbofno_layer_2d_workspace_bytes.restype = sz
         L.turbofno_layer_2d.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, vp, sz, i, vp]
+        L.turbofno_fft2d_trunc.argtypes = [i, i, vp, vp, l, vp]
+        L.turbofno_ifft2d_pad.argtypes = [i, i, vp, vp, l, vp]
+        L.turbofno_cgemm.argtypes = [l, i, i, vp, vp, vp, f, f, vp]
         L.turbofno_last_error_string.restype = ctypes.c_char_p
         L.turbofno_abi_version.restype = i
         for name in ("turbofno_fused_fft_cgemm_ifft", "turbofno_fft_stride", "turbofno_ifft_stride",
-                     "turbofno_layer_1d", "turbofno_layer_2d"):
+                     "turbofno_layer_1d", "turbofno_layer_2d", "turbofno_fft2d_trunc", "turbofno_ifft2d_pad",
+                     "turbofno_cgemm"):
             getattr(L, name).restype = i
         _LIB = L
     return _LIB
@@ -127,3 +131,27 @@ def layer_2d(x, W, y=None, alpha=1.0 + 0j, workspace=None, algo=0):
     _check(lib().turbofno_layer_2d(bs, DX, DY, K, N, _dev_c64(x, "x"), _dev_c64(W, "W"), _dev_c64(y, "y"),
                                    a.real, a.imag, workspace.data_ptr(), workspace.numel(), algo, _stream()))
     return y
+
+
+def fft2d_trunc(x, spec):
+    """x: [nimg][256][256] -> spec: [nimg][4096] (retained 64 x 64 modes, kernel-private order)."""
+    nimg = x.numel() // (x.shape[-1] * x.shape[-2])
+    _check(lib().turbofno_fft2d_trunc(x.shape[-2], x.shape[-1], _dev_c64(x, "x"), _dev_c64(spec, "spec"), nimg,
+                                      _stream()))
+    return spec
+
+
+def ifft2d_pad(spec, y):
+    """spec: [nimg][4096] -> y: [nimg][256][256]."""
+    nimg = y.numel() // (y.shape[-1] * y.shape[-2])
+    _check(lib().turbofno_ifft2d_pad(y.shape[-2], y.shape[-1], _dev_c64(spec, "spec"), _dev_c64(y, "y"), nimg,
+                                     _stream()))
+    return y
+
+
+def cgemm(M, N, K, A, B, C, alpha=1.0 + 0j):
+    """C[m + n*M] = alpha * sum_k A[m + k*M] B[k + n*K]  (A: [K][M], B: [N][K], C: [N][M] as tensors)."""
+    a = complex(alpha)
+    _check(lib().turbofno_cgemm(M, N, K, _dev_c64(A, "A"), _dev_c64(B, "B"), _dev_c64(C, "C"), a.real, a.imag,
+                                _stream()))
+    return C

@@ -101,6 +101,31 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
     return turbofno_fused_fft_cgemm_ifft(logDY, (long)bs * dimX * 64, N, K, x, W, nullptr, y, alpha_re, alpha_im, 0.f, 0.f, stream);
 }
 
+int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream)
+{
+    if (!x || !spec) return fail(TURBOFNO_ERR_INVALID_ARG, "x and spec must be non-null device pointers");
+    if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
+    if (DX != 256 || DY != 256) return fail(TURBOFNO_ERR_UNSUPPORTED, "whole-image transforms are built for DX = DY = 256 only");
+    return hip_status(tfno::launch_fft2d_trunc_256((const float2*)x, (float2*)spec, nimg, (hipStream_t)stream), "fft2d_trunc launch");
+}
+
+int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, void* stream)
+{
+    if (!spec || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "spec and y must be non-null device pointers");
+    if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
+    if (DX != 256 || DY != 256) return fail(TURBOFNO_ERR_UNSUPPORTED, "whole-image transforms are built for DX = DY = 256 only");
+    return hip_status(tfno::launch_ifft2d_pad_256((const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
+}
+
+int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im, void* stream)
+{
+    if (!A || !B || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "A, B and C must be non-null device pointers");
+    if (int rc = check_gemm_dims(M, N, K)) return rc;
+    if (M % 128) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld is not a multiple of the 128-row block tile", M);
+    return hip_status(tfno::launch_cgemm_modes((const float2*)A, (const float2*)B, (float2*)C, M, N, K,
+                                               make_float2(alpha_re, alpha_im), (hipStream_t)stream), "cgemm launch");
+}
+
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
