@@ -1,0 +1,58 @@
+"""Host drivers: config grammar (CPU) and the result-line format of the executables (GPU)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def config_check(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("host") / "config_check")
+    subprocess.run(["hipcc", "-O1", "-std=c++17", os.path.join(ROOT, "tests", "host", "config_check.cpp"),
+                    os.path.join(ROOT, "turbofno_amd", "host", "utils.cpp"), "-o", exe], check=True,
+                   stderr=subprocess.DEVNULL)
+    return exe
+
+
+def run_cfg(exe, path):
+    return subprocess.run([exe, path], check=True, capture_output=True, text=True).stdout.strip()
+
+
+def test_config_grammar(config_check, tmp_path):
+    # grammar of the reference's benchmark_config/*.txt: "key = v v v", '#' comments, blank lines,
+    # last line without trailing newline (utils/utils.cu:14-22, fused.cu:84-90)
+    p = tmp_path / "cfg.txt"
+    p.write_text("# comment\n\nbs_list = 1 2 4\nDX_list = 128 256\nK_list = 8 16 24 32 40\nN_list = 64")
+    assert run_cfg(config_check, str(p)) == "DX_list:128,256;K_list:8,16,24,32,40;N_list:64;bs_list:1,2,4;"
+    # a missing file gives zero problems, as in the reference
+    assert run_cfg(config_check, str(tmp_path / "missing.txt")) == ""
+
+
+def test_shipped_configs_parse(config_check):
+    out = run_cfg(config_check, os.path.join(ROOT, "benchmark_config", "problem_size_1d.txt"))
+    assert "dimX_list:1;" in out and "DY_list:128,256;" in out and "K_list:8,16,24,32;" in out
+    out = run_cfg(config_check, os.path.join(ROOT, "benchmark_config", "problem_size_2d.txt"))
+    assert "DX_list:128,256;" in out and "bs_list:1,4,16;" in out
+
+
+@pytest.mark.gpu
+def test_driver_result_lines():
+    exe1, exe2 = os.path.join(ROOT, "bin", "TurboFNO_1D_D"), os.path.join(ROOT, "bin", "TurboFNO_2D_D")
+    assert os.path.exists(exe1) and os.path.exists(exe2), "build the drivers with make -C turbofno_amd/host"
+    out = subprocess.run([exe1, "4", "1", "128", "64", "16"], check=True, capture_output=True, text=True, timeout=100).stdout
+    print(out, flush=True)
+    assert re.fullmatch(r"1D_D, bs=4   , dimX=1   , DY=128 , N=64  , K=16  , TIME=\s*\d+\.\d{3}ms\n", out), out
+    out = subprocess.run([exe2, "1", "256", "256", "64", "16"], check=True, capture_output=True, text=True, timeout=100).stdout
+    print(out, flush=True)
+    assert re.fullmatch(r"2D_D, bs=1   , DX=256 , DY=256 , N=64  , K=16  , TIME=\s*\d+\.\d{3}ms\n", out), out
+    # config-file mode: a tiny grid, loop order bs -> DX -> DY -> N -> K
+    cfg = os.path.join(ROOT, "gpurun_out", "tiny_2d.txt")
+    os.makedirs(os.path.dirname(cfg), exist_ok=True)
+    with open(cfg, "w") as f:
+        f.write("bs_list = 1\nDX_list = 128 256\nDY_list = 128\nN_list = 64\nK_list = 8 16")
+    lines = subprocess.run([exe2, cfg], check=True, capture_output=True, text=True, timeout=100).stdout.splitlines()
+    got = [tuple(int(v) for v in re.findall(r"=(\d+)", ln)[:5]) for ln in lines]
+    assert got == [(1, 128, 128, 64, 8), (1, 128, 128, 64, 16), (1, 256, 128, 64, 8), (1, 256, 128, 64, 16)], lines

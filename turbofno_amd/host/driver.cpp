@@ -1,0 +1,110 @@
+// Drivers TurboFNO_1D_D and TurboFNO_2D_D: the fully fused 1D / 2D spectral layer, timed per problem.
+//
+// Surface kept from the reference (fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:20-151,
+// fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:33-208):
+//   * problems come from benchmark_config/problem_size_{1d,2d}.txt (DEFAULT_CONFIG_PATH baked in at
+//     build time), loop order bs -> dimX|DX -> DY -> N -> K;
+//   * alternatively five positional integers "<bs> <dimX|DX> <DY> <N> <K>" run a single problem
+//     (fusion_variants_benchmark/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:33-46), or one argument
+//     names another config file (documented at README.md:122-132);
+//   * inputs: +-{0..9}e-3 from rand(); alpha = (1,-1);
+//   * timing: one warm-up, then ntest x (launch + device synchronise) between two events, mean;
+//   * one result line per problem, format identical to fused.cu:146-147 / fused_trunc_2D.cu:203-204.
+// Differences: device buffers are sized per problem (the reference allocates once for its largest
+// hard-coded problem); the kernels are reached through the C ABI of include/turbofno.h.
+#include "../../include/turbofno.h"
+#include "TurboFNO.h"
+#include "utils.h"
+#include <cstring>
+#include <string>
+
+#ifndef TURBOFNO_VARIANT_2D
+#define TURBOFNO_VARIANT_2D 0
+#endif
+#ifndef DEFAULT_CONFIG_PATH
+#define DEFAULT_CONFIG_PATH "benchmark_config/problem_size_1d.txt"
+#endif
+
+struct Problem { int bs, dx, dy, n, k; };
+
+static std::vector<Problem> problems_from(int argc, char** argv)
+{
+    std::vector<Problem> out;
+    if (argc == 6) {
+        out.push_back({ atoi(argv[1]), atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]) });
+        return out;
+    }
+    auto cfg = load_problem_config(argc == 2 ? argv[1] : DEFAULT_CONFIG_PATH);
+    const char* xkey = TURBOFNO_VARIANT_2D ? "DX_list" : "dimX_list";
+    for (int bs : cfg["bs_list"])
+        for (int dx : cfg[xkey])
+            for (int dy : cfg["DY_list"])
+                for (int n : cfg["N_list"])
+                    for (int k : cfg["K_list"]) out.push_back({ bs, dx, dy, n, k });
+    return out;
+}
+
+int main(int argc, char** argv)
+{
+    const float alpha_re = 1.0f, alpha_im = -1.0f;
+    int algo = TURBOFNO_2D_AUTO;
+    if (const char* e = getenv("TURBOFNO_2D_ALGO")) algo = atoi(e);
+    if (const char* e = getenv("TURBOFNO_NTEST")) ntest = atoi(e) > 0 ? atoi(e) : ntest;
+
+    for (const Problem& p : problems_from(argc, argv)) {
+        // 1D: x[K][bs*dimX][DY]; 2D: x[K][bs][DX][DY]
+        const size_t per_channel = TURBOFNO_VARIANT_2D ? (size_t)p.bs * p.dx * p.dy : (size_t)p.bs * p.dx * p.dy;
+        const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
+        float* hx = (float*)malloc(sizeof(float) * 2 * in_elems);
+        float* hw = (float*)malloc(sizeof(float) * 2 * w_elems);
+        generate_random_vector(hx, 2 * (long)in_elems);
+        generate_random_vector(hw, 2 * (long)w_elems);
+        void *dx = nullptr, *dw = nullptr, *dy = nullptr, *dws = nullptr;
+        HIP_RT_CALL(hipMalloc(&dx, sizeof(float) * 2 * in_elems));
+        HIP_RT_CALL(hipMalloc(&dw, sizeof(float) * 2 * w_elems));
+        HIP_RT_CALL(hipMalloc(&dy, sizeof(float) * 2 * out_elems));
+        HIP_RT_CALL(hipMemcpy(dx, hx, sizeof(float) * 2 * in_elems, hipMemcpyHostToDevice));
+        HIP_RT_CALL(hipMemcpy(dw, hw, sizeof(float) * 2 * w_elems, hipMemcpyHostToDevice));
+        size_t ws_bytes = 0;
+        if (TURBOFNO_VARIANT_2D) {
+            ws_bytes = turbofno_layer_2d_workspace_bytes(p.bs, p.dx, p.dy, p.k, p.n, algo);
+            HIP_RT_CALL(hipMalloc(&dws, ws_bytes ? ws_bytes : 256));
+        }
+        auto launch = [&]() {
+            if (TURBOFNO_VARIANT_2D)
+                CHECK_TURBOFNO(turbofno_layer_2d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, dws, ws_bytes, algo, nullptr));
+            else
+                CHECK_TURBOFNO(turbofno_layer_1d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, nullptr));
+        };
+        HIP_RT_CALL(hipDeviceSynchronize());
+        launch();
+        CHECK_HIP_KERNEL();
+        HIP_RT_CALL(hipDeviceSynchronize());
+        CHECK_HIP_KERNEL();
+
+        hipEvent_t t_begin, t_end;
+        float elapsed_time = 0.f;
+        HIP_RT_CALL(hipEventCreate(&t_begin));
+        HIP_RT_CALL(hipEventCreate(&t_end));
+        HIP_RT_CALL(hipEventRecord(t_begin));
+        for (int i = 0; i < ntest; ++i) {
+            launch();
+            HIP_RT_CALL(hipDeviceSynchronize());
+        }
+        HIP_RT_CALL(hipEventRecord(t_end));
+        HIP_RT_CALL(hipEventSynchronize(t_end));
+        HIP_RT_CALL(hipEventElapsedTime(&elapsed_time, t_begin, t_end));
+        elapsed_time /= ntest;
+        if (TURBOFNO_VARIANT_2D)
+            printf("2D_D, bs=%-4d, DX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
+        else
+            printf("1D_D, bs=%-4d, dimX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
+        fflush(stdout);
+        HIP_RT_CALL(hipEventDestroy(t_begin));
+        HIP_RT_CALL(hipEventDestroy(t_end));
+        HIP_RT_CALL(hipFree(dx)); HIP_RT_CALL(hipFree(dw)); HIP_RT_CALL(hipFree(dy));
+        if (dws) HIP_RT_CALL(hipFree(dws));
+        free(hx); free(hw);
+    }
+    return 0;
+}

@@ -1,0 +1,47 @@
+// Host-side helpers of the drivers: config-file grammar, random fill, HIP error checks.
+// Counterparts in the reference: utils/utils.cu:14-22 (parse_line), :37-43 (generate_random_vector),
+// utils/utils.cuh:17-25 (kernel check that exits), :43-57 (runtime-call check that only prints).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <string>
+#include <vector>
+
+// values of one "key = v v v" line (the first two tokens are skipped)
+std::vector<int> parse_line(const std::string& line);
+
+// whole file -> key -> values; '#' comments and blank lines are skipped; a missing file yields an
+// empty map (the reference's unchecked ifstream behaves the same: zero problems are run)
+std::map<std::string, std::vector<int>> load_problem_config(const std::string& path);
+
+// +-{0..9} * 1e-3 from rand(), unseeded: the reference's input distribution
+void generate_random_vector(float* target, long n);
+
+#define HIP_RT_CALL(call)                                                                                    \
+    do {                                                                                                     \
+        hipError_t status_ = (call);                                                                         \
+        if (status_ != hipSuccess)                                                                           \
+            fprintf(stderr, "HIP runtime error at %s:%d: %s (%d)\n", __FILE__, __LINE__,                     \
+                    hipGetErrorString(status_), (int)status_);                                               \
+    } while (0)
+
+#define CHECK_HIP_KERNEL()                                                                                   \
+    do {                                                                                                     \
+        hipError_t status_ = hipGetLastError();                                                              \
+        if (status_ != hipSuccess) {                                                                         \
+            fprintf(stderr, "kernel error at %s:%d: %s\n", __FILE__, __LINE__, hipGetErrorString(status_)); \
+            exit(EXIT_FAILURE);                                                                              \
+        }                                                                                                    \
+    } while (0)
+
+#define CHECK_TURBOFNO(call)                                                                                 \
+    do {                                                                                                     \
+        int rc_ = (call);                                                                                    \
+        if (rc_ != 0) {                                                                                      \
+            fprintf(stderr, "turbofno error %d at %s:%d: %s\n", rc_, __FILE__, __LINE__,                     \
+                    turbofno_last_error_string());                                                           \
+            exit(EXIT_FAILURE);                                                                              \
+        }                                                                                                    \
+    } while (0)
