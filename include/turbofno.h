@@ -97,7 +97,7 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
  *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] (column major, lda = M, ldb = K,
  *   ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
  *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:182-200) for beta = 0,
- *   the only value with which the fused variant D uses the product. Requires M % 128 == 0, N % 64 == 0,
+ *   the only value with which the fused variant D uses the product. Requires M % 256 == 0, N % 64 == 0,
  *   K % 8 == 0.
  */
 int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream);

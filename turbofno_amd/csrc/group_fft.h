@@ -17,14 +17,12 @@ template <int LOGDY> struct Geo1D {
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * 64 + GROUPS * EXCH);
 };
 
-// forward transform of one signal by one L-lane group; lane t holds samples t + L*i in v[].
-// On return lane `t` holds modes m = t + L*mm in out[mm].
+// second half of the forward transform: exchange of the twiddled first-pass results g[] inside the
+// L-lane group, then the pruned L-point DFT. On return lane `t` holds modes m = t + L*mm in out[mm].
 template <int LOGDY>
-TFNO_DEV void group_forward(cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
+TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
 {
     constexpr int L = Geo1D<LOGDY>::L;
-    cpx g[16];
-    fwd_pass1(v, tw, g);
     wave_lds_fence();
 #pragma unroll
     for (int r = 0; r < 16; ++r) exch[t * 17 + r] = g[r];
@@ -43,6 +41,16 @@ TFNO_DEV void group_forward(cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t,
 #pragma unroll
         for (int s = 0; s < 4; ++s) { out[2 * s] = o0[s]; out[2 * s + 1] = o1[s]; }
     }
+}
+
+// forward transform of one signal by one L-lane group; lane t holds samples t + L*i in v[].
+// On return lane `t` holds modes m = t + L*mm in out[mm].
+template <int LOGDY>
+TFNO_DEV void group_forward(cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
+{
+    cpx g[16];
+    fwd_pass1(v, tw, g);
+    group_forward_finish<LOGDY>(g, exch, t, out);
 }
 
 // zero-padded backward transform; lane t holds modes m = t + L*mm in c[]; returns samples t + L*i in y[].

@@ -26,50 +26,81 @@ constexpr int IMG = 256;
 constexpr int TPITCH = 66;                       // row pitch (complex) of the 256 x 64 redistribution tile
 constexpr int EXCH256 = 16 * 17;                 // exchange region of one 16-lane group
 constexpr size_t LDS2D_BYTES = sizeof(float2) * (size_t)(64 * EXCH256 > IMG * TPITCH ? 64 * EXCH256 : IMG * TPITCH);
+constexpr size_t LDS2D_FWD_BYTES = sizeof(float2) * (size_t)(IMG * TPITCH);   // 32 groups: tile is the larger user
 
-// Row handled by 16-lane group j of wave w in pass `it`: groups 0/1 of a wave are 8 rows apart so the
-// two groups that share an LDS cycle hit disjoint banks in the pitch-66 tile.
+// Row handled by 16-lane group j of wave w in pass `it` (64 groups per block): groups 0/1 of a wave are
+// 8 rows apart so the two groups that share an LDS cycle hit disjoint banks in the pitch-66 tile.
 __device__ __forceinline__ int row_of(int w, int j, int it)
 {
     return 64 * it + ((w & 7) | ((j & 1) << 3) | ((j >> 1) << 4) | ((w >> 3) << 5));
 }
+// same for a 512-thread block (32 groups, 8 passes)
+__device__ __forceinline__ int row_of32(int w, int j, int it)
+{
+    return 32 * it + (w | ((j & 1) << 3) | ((j >> 1) << 4));
+}
 }  // namespace
 
-__global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec)
+// Forward image kernel. 512 threads = 32 lane groups; a block is persistent over images
+// (img = blockIdx.x, += gridDim.x) and keeps two rows per group in flight ahead of the arithmetic,
+// across pass 2 and across image boundaries, so HBM reads never pause while the columns are transformed.
+__global__ __launch_bounds__(512) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
+                                                              int nimg)
 {
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
-    const long img = blockIdx.x;
     float2* exch = lds + g * EXCH256;
 
     cpx tw[16];
     load_lane_twiddles<8>(r, tw);
 
-    // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row_of(w, j, it)
-    cpx T[4][4];
+    const int row0 = row_of32(w, j, 0);
+    auto issue = [&](cpx (&dst)[16], long img, int it) {
+        const float2* src = x + (img * IMG + row0 + 32 * it) * IMG + r;
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        const float2* src = x + (img * IMG + row_of(w, j, it)) * IMG + r;
-        cpx v[16];
+        for (int i = 0; i < 16; ++i) dst[i] = src[16 * i];
+    };
+
+    long img = blockIdx.x;
+    cpx va[16], vb[16];
+    if (img < nimg) { issue(va, img, 0); issue(vb, img, 1); }
+    for (; img < nimg; img += gridDim.x) {
+        const long nxt = img + gridDim.x;
+        // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 32 it
+        cpx T[8][4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = src[16 * i];
-        group_forward<8>(v, tw, exch, r, T[it]);
+        for (int it = 0; it < 8; it += 2) {
+            cpx ga[16], gb[16];
+            fwd_pass1(va, tw, ga);
+            if (it + 2 < 8) issue(va, img, it + 2);
+            group_forward_finish<8>(ga, exch, r, T[it]);
+            fwd_pass1(vb, tw, gb);
+            if (it + 3 < 8) issue(vb, img, it + 3);
+            group_forward_finish<8>(gb, exch, r, T[it + 1]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 8; ++it)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) lds[(row0 + 32 * it) * TPITCH + r + 16 * s] = T[it][s];
+        __syncthreads();
+        // pass 2: columns (along X); group g owns columns q = g and g + 32, lane r holds rows r + 16 i
+        cpx c0[16], c1[16], z0[4], z1[4];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            c0[i] = lds[(r + 16 * i) * TPITCH + g];
+            c1[i] = lds[(r + 16 * i) * TPITCH + g + 32];
+        }
+        __syncthreads();
+        // the row registers are free again: start the next image's first rows before the column pass
+        if (nxt < nimg) { issue(va, nxt, 0); issue(vb, nxt, 1); }
+        group_forward<8>(c0, tw, exch, r, z0);
+        group_forward<8>(c1, tw, exch, r, z1);
+        // lane order of the retained modes: element s*1024 + q*16 + r  <->  mode (p = r + 16 s, q)
+        float2* dst = spec + img * 4096 + g * 16 + r;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { dst[1024 * s] = z0[s]; dst[1024 * s + 512] = z1[s]; }
     }
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < 4; ++it)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) lds[row_of(w, j, it) * TPITCH + r + 16 * s] = T[it][s];
-    __syncthreads();
-    // pass 2: columns (along X); group g owns column q = g, lane r holds rows r + 16 i
-    cpx v[16], z[4];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) v[i] = lds[(r + 16 * i) * TPITCH + g];
-    __syncthreads();
-    group_forward<8>(v, tw, exch, r, z);
-    float2* dst = spec + img * 4096 + tid;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) dst[1024 * s] = z[s];
 }
 
 __global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __restrict__ spec, float2* __restrict__ y)
@@ -122,15 +153,18 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __re
 // ---------------------------------------------------------------------------------------------
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int GEMM_KC = 64;      // channels per LDS-resident W chunk
+constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
+constexpr int GEMM_WPITCH = 260;    // floats per k row of the W tile (256 + 4: spreads the k-major fill over banks)
+constexpr int GEMM_THREADS = 512;   // 8 waves, one 32-m strip each -> 256 m per block
 
-__global__ __launch_bounds__(256) void cgemm_modes_kernel(const float2* __restrict__ A, const float2* __restrict__ W,
-                                                          float2* __restrict__ C, long Mtot, int N, int K, float2 alpha)
+__global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
+                                                                   const float2* __restrict__ W, float2* __restrict__ C,
+                                                                   long Mtot, int N, int K, float2 alpha)
 {
-    // sW[(k*128 + n')*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:  {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1
-    __shared__ float sW[GEMM_KC * 128 * 2];
+    // sW[k*260 + n'*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:  {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1
+    __shared__ float sW[GEMM_KC * GEMM_WPITCH];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
-    const long m0 = ((long)blockIdx.x * 4 + wave) * 32;
+    const long m0 = ((long)blockIdx.x * (GEMM_THREADS / 64) + wave) * 32;
     const int n0 = blockIdx.y * 64;
 
     floatx16 acc[4];
@@ -141,27 +175,31 @@ __global__ __launch_bounds__(256) void cgemm_modes_kernel(const float2* __restri
 
     for (int kc = 0; kc < K; kc += GEMM_KC) {
         const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;
+        // lane (col, half) feeds A[kc + kk + half][m0 + col] as {re, im}; all loads of the chunk are issued
+        // before the W tile is built so their latency hides behind it
+        const float2* ap = A + (long)(kc + half) * Mtot + m0 + col;
+        float2 bv[GEMM_KC / 2];
+#pragma unroll
+        for (int q = 0; q < GEMM_KC / 2; ++q)
+            bv[q] = (2 * q < kn) ? ap[(long)(2 * q) * Mtot] : make_float2(0.f, 0.f);
         __syncthreads();
-        for (int idx = tid; idx < GEMM_KC * 64; idx += 256) {
-            int n = idx % 64, k = idx / 64;   // n fastest: conflict-free 16 B LDS stores
+        for (int idx = tid; idx < GEMM_KC * 64; idx += GEMM_THREADS) {
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;   // k fastest: coalesced reads of W[k + n*K]
             float2 w = make_float2(0.f, 0.f);
             if (k < kn) {
                 float2 w0 = W[(kc + k) + (long)(n0 + n) * K];
                 w = make_float2(w0.x * alpha.x - w0.y * alpha.y, w0.x * alpha.y + w0.y * alpha.x);
             }
-            *reinterpret_cast<float4*>(&sW[(k * 128 + 2 * n) * 2]) = make_float4(w.x, -w.y, w.y, w.x);
+            *reinterpret_cast<float4*>(&sW[k * GEMM_WPITCH + 4 * n]) = make_float4(w.x, -w.y, w.y, w.x);
         }
         __syncthreads();
-        // lane (col, half) feeds A[kc + kk + half][m0 + col] as {re, im}: two contraction steps
-        const float2* ap = A + (long)(kc + half) * Mtot + m0 + col;
-#pragma unroll 4
-        for (int kk = 0; kk < kn; kk += 2) {
-            float2 b = ap[(long)kk * Mtot];
+#pragma unroll
+        for (int q = 0; q < GEMM_KC / 2; ++q) {
 #pragma unroll
             for (int tI = 0; tI < 4; ++tI) {
-                float2 a = *reinterpret_cast<const float2*>(&sW[((kk + half) * 128 + tI * 32 + col) * 2]);
-                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc[tI], 0, 0, 0);
-                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc[tI], 0, 0, 0);
+                float2 a = *reinterpret_cast<const float2*>(&sW[(2 * q + half) * GEMM_WPITCH + (tI * 32 + col) * 2]);
+                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bv[q].x, acc[tI], 0, 0, 0);
+                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bv[q].y, acc[tI], 0, 0, 0);
             }
         }
     }
@@ -177,16 +215,31 @@ __global__ __launch_bounds__(256) void cgemm_modes_kernel(const float2* __restri
             }
 }
 
+static int cu_count()
+{
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        else cus = 256;
+    }
+    return cus;
+}
+
 hipError_t launch_fft2d_trunc_256(const float2* x, float2* spec, long nimg, hipStream_t stream)
 {
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fft2d_trunc_256_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_FWD_BYTES);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)nimg), dim3(1024), LDS2D_BYTES, stream, x, spec);
+    // one persistent block per CU (the LDS tile allows exactly one resident block per CU)
+    const long blocks = nimg < cu_count() ? nimg : cu_count();
+    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)blocks), dim3(512), LDS2D_FWD_BYTES, stream, x, spec,
+                       (int)nimg);
     return hipGetLastError();
 }
 
@@ -206,9 +259,9 @@ hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipSt
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               hipStream_t stream)
 {
-    if (Mtot % 128 != 0 || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
-    dim3 grid((unsigned)(Mtot / 128), (unsigned)(N / 64), 1);
-    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(256), 0, stream, A, W, C, Mtot, N, K, alpha);
+    if (Mtot % 256 != 0 || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(Mtot / 256), (unsigned)(N / 64), 1);
+    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha);
     return hipGetLastError();
 }
 
