@@ -107,6 +107,27 @@ template <int DIR> TFNO_DEV void fft16(cpx (&v)[16])
     for (int rho = 0; rho < 4; ++rho) radix4<DIR>(v[4 * rho], v[4 * rho + 1], v[4 * rho + 2], v[4 * rho + 3]);
 }
 
+// The same transform in two steps, out of place: fft16_stage1 reads v[] and leaves the first radix-4
+// stage (twiddled) in b[]; after it v[] is dead, so the caller can reuse those registers (e.g. as the
+// landing zone of the next row's loads) while fft16_stage2 finishes in b[].
+template <int DIR> TFNO_DEV void fft16_stage1(const cpx (&v)[16], cpx (&b)[16])
+{
+#pragma unroll
+    for (int i0 = 0; i0 < 4; ++i0) {
+        cpx a0 = v[i0], a1 = v[i0 + 4], a2 = v[i0 + 8], a3 = v[i0 + 12];
+        radix4<DIR>(a0, a1, a2, a3);
+        b[i0] = a0; b[i0 + 4] = a1; b[i0 + 8] = a2; b[i0 + 12] = a3;
+    }
+    b[5] = mul_w16<DIR, 1>(b[5]);   b[9] = mul_w16<DIR, 2>(b[9]);   b[13] = mul_w16<DIR, 3>(b[13]);
+    b[6] = mul_w16<DIR, 2>(b[6]);   b[10] = mul_w16<DIR, 4>(b[10]); b[14] = mul_w16<DIR, 6>(b[14]);
+    b[7] = mul_w16<DIR, 3>(b[7]);   b[11] = mul_w16<DIR, 6>(b[11]); b[15] = mul_w16<DIR, 9>(b[15]);
+}
+template <int DIR> TFNO_DEV void fft16_stage2(cpx (&b)[16])
+{
+#pragma unroll
+    for (int rho = 0; rho < 4; ++rho) radix4<DIR>(b[4 * rho], b[4 * rho + 1], b[4 * rho + 2], b[4 * rho + 3]);
+}
+
 // First four bins (s = 0..3) of a 16-point DFT of g[0..15]:  out[s] = sum_t g[t] w16^(t s).
 template <int DIR> TFNO_DEV void dft16_first4(cpx (&g)[16], cpx (&out)[4])
 {
@@ -171,6 +192,65 @@ template <int LOGD> TFNO_DEV void load_lane_twiddles(int t, cpx (&tw)[16])
 {
 #pragma unroll
     for (int r = 0; r < 16; ++r) tw[r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
+}
+
+// Inter-pass twiddles kept in LDS instead of registers (frees 30 VGPRs for kernels that run 16 waves
+// per CU). Table layout: tab[t*18 + r] = w_D^(t r), t < 16 lanes, r < 16; the pitch of 18 complex keeps
+// 16-byte alignment for ds_read_b128 and spreads the 16 lanes of a group over all 64 banks.
+constexpr int kTwLdsPitch = 18;
+constexpr int kTwLdsSize = 16 * kTwLdsPitch;   // complex elements
+
+#ifndef TFNO_HOST_CHECK
+template <int LOGD> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
+{
+    for (int e = tid; e < 256; e += nthreads) {
+        const int t = e >> 4, r = e & 15;
+        tab[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
+    }
+}
+#endif
+
+// Forward first pass with LDS twiddles: row = tab + t*kTwLdsPitch for lane t.
+TFNO_DEV void fwd_pass1_lds(cpx (&v)[16], const cpx* row, cpx (&g)[16])
+{
+    fft16<-1>(v);
+    g[0] = v[0];
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) {
+        const float4 w = *reinterpret_cast<const float4*>(row + r);      // tw[r], tw[r+1]
+        g[r] = cmul(v[fft16_slot(r)], make_float2(w.x, w.y));
+        g[r + 1] = cmul(v[fft16_slot(r + 1)], make_float2(w.z, w.w));
+    }
+    g[1] = cmul(v[fft16_slot(1)], row[1]);
+}
+
+// Second half of fwd_pass1_lds for a caller that ran fft16_stage1 itself: b[] in, twiddled bins out in g[].
+TFNO_DEV void fwd_pass1_lds_finish(cpx (&b)[16], const cpx* row, cpx (&g)[16])
+{
+    fft16_stage2<-1>(b);
+    g[0] = b[0];
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) {
+        const float4 w = *reinterpret_cast<const float4*>(row + r);      // tw[r], tw[r+1]
+        g[r] = cmul(b[fft16_slot(r)], make_float2(w.x, w.y));
+        g[r + 1] = cmul(b[fft16_slot(r + 1)], make_float2(w.z, w.w));
+    }
+    g[1] = cmul(b[fft16_slot(1)], row[1]);
+}
+
+// Backward last pass with LDS twiddles.
+TFNO_DEV void inv_pass2_lds(cpx (&e)[16], const cpx* row, cpx (&y)[16])
+{
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) {
+        const float4 w = *reinterpret_cast<const float4*>(row + r);
+        e[r] = cmulc(e[r], make_float2(w.x, w.y));
+        e[r + 1] = cmulc(e[r + 1], make_float2(w.z, w.w));
+    }
+    e[1] = cmulc(e[1], row[1]);
+    fft16<+1>(e);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = e[fft16_slot(i)];
 }
 
 // Forward first pass: 16-point FFT of the lane's strided samples, then the inter-pass twiddle.

@@ -80,4 +80,19 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
     inv_pass2(e, tw, y);
 }
 
+// zero-padded backward transform (L = 16) whose last pass takes its twiddles from an LDS table row.
+TFNO_DEV void group_backward256_lds(const cpx (&c)[4], const cpx* twrow, cpx* exch, int t, cpx (&y)[16])
+{
+    wave_lds_fence();
+    cpx h[16];
+    dft16_pad4<+1>(c, h);
+#pragma unroll
+    for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+    wave_lds_fence();
+    cpx e[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+    inv_pass2_lds(e, twrow, y);
+}
+
 }  // namespace tfno

@@ -25,8 +25,9 @@ namespace {
 constexpr int IMG = 256;
 constexpr int TPITCH = 66;                       // row pitch (complex) of the 256 x 64 redistribution tile
 constexpr int EXCH256 = 16 * 17;                 // exchange region of one 16-lane group
-constexpr size_t LDS2D_BYTES = sizeof(float2) * (size_t)(64 * EXCH256 > IMG * TPITCH ? 64 * EXCH256 : IMG * TPITCH);
-constexpr size_t LDS2D_FWD_BYTES = sizeof(float2) * (size_t)(IMG * TPITCH);   // 32 groups: tile is the larger user
+constexpr int LDS2D_ELEMS = 64 * EXCH256 > IMG * TPITCH ? 64 * EXCH256 : IMG * TPITCH;   // exchange regions alias the tile
+constexpr size_t LDS2D_BYTES = sizeof(float2) * (size_t)LDS2D_ELEMS;
+constexpr size_t LDS2D_FWD_BYTES = sizeof(float2) * (size_t)(LDS2D_ELEMS + kTwLdsSize);
 
 // Row handled by 16-lane group j of wave w in pass `it` (64 groups per block): groups 0/1 of a wave are
 // 8 rows apart so the two groups that share an LDS cycle hit disjoint banks in the pitch-66 tile.
@@ -41,65 +42,77 @@ __device__ __forceinline__ int row_of32(int w, int j, int it)
 }
 }  // namespace
 
-// Forward image kernel. 512 threads = 32 lane groups; a block is persistent over images
-// (img = blockIdx.x, += gridDim.x) and keeps two rows per group in flight ahead of the arithmetic,
-// across pass 2 and across image boundaries, so HBM reads never pause while the columns are transformed.
-__global__ __launch_bounds__(512) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
-                                                              int nimg)
+// Forward image kernel. 1024 threads = 64 lane groups = 16 waves per CU (4 per SIMD: the arithmetic
+// is issue bound, so full occupancy matters more than registers). A block is persistent over images
+// (img = blockIdx.x, += gridDim.x). Each group keeps ONE row in flight: the loads of its next row are
+// issued as soon as the first pass has consumed the row registers, so they travel while the exchange
+// and the second pass run, across the column pass and across image boundaries. Inter-pass twiddles
+// live in LDS to keep the kernel at 128 VGPRs.
+__global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
+                                                               int nimg)
 {
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
     float2* exch = lds + g * EXCH256;
+    float2* twtab = lds + LDS2D_ELEMS;                 // after the exchange regions / tile
+    fill_lds_twiddles<8>(twtab, tid, 1024);
+    const float2* twrow = twtab + r * kTwLdsPitch;
+    __syncthreads();
 
-    cpx tw[16];
-    load_lane_twiddles<8>(r, tw);
-
-    const int row0 = row_of32(w, j, 0);
+    const int row0 = row_of(w, j, 0);
+    // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
+    const unsigned lane_off = (unsigned)(row0 * IMG + r);
     auto issue = [&](cpx (&dst)[16], long img, int it) {
-        const float2* src = x + (img * IMG + row0 + 32 * it) * IMG + r;
+        const float2* base = x + (img * IMG + 64 * it) * (long)IMG;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = src[16 * i];
+        for (int i = 0; i < 16; ++i) dst[i] = base[lane_off + 16u * i];
     };
 
     long img = blockIdx.x;
-    cpx va[16], vb[16];
-    if (img < nimg) { issue(va, img, 0); issue(vb, img, 1); }
+    cpx v[16];
+    if (img < nimg) issue(v, img, 0);
     for (; img < nimg; img += gridDim.x) {
         const long nxt = img + gridDim.x;
-        // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 32 it
-        cpx T[8][4];
+        // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 64 it
+        cpx T[4][4];
 #pragma unroll
-        for (int it = 0; it < 8; it += 2) {
-            cpx ga[16], gb[16];
-            fwd_pass1(va, tw, ga);
-            if (it + 2 < 8) issue(va, img, it + 2);
-            group_forward_finish<8>(ga, exch, r, T[it]);
-            fwd_pass1(vb, tw, gb);
-            if (it + 3 < 8) issue(vb, img, it + 3);
-            group_forward_finish<8>(gb, exch, r, T[it + 1]);
+        for (int it = 0; it < 4; ++it) {
+            cpx bb[16], gg[16];
+            fft16_stage1<-1>(v, bb);
+            // v is dead after the first radix-4 stage: its registers become the landing zone of the next row
+            if (it + 1 < 4) issue(v, img, it + 1);
+            fwd_pass1_lds_finish(bb, twrow, gg);
+            group_forward_finish<8>(gg, exch, r, T[it]);
         }
         __syncthreads();
 #pragma unroll
-        for (int it = 0; it < 8; ++it)
+        for (int it = 0; it < 4; ++it)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) lds[(row0 + 32 * it) * TPITCH + r + 16 * s] = T[it][s];
+            for (int s = 0; s < 4; ++s) lds[(row0 + 64 * it) * TPITCH + r + 16 * s] = T[it][s];
         __syncthreads();
-        // pass 2: columns (along X); group g owns columns q = g and g + 32, lane r holds rows r + 16 i
-        cpx c0[16], c1[16], z0[4], z1[4];
+        // pass 2: columns (along X); group g owns column q = g, lane r holds rows r + 16 i
+        cpx z[4];
+        {
+            cpx c[16], gg[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            c0[i] = lds[(r + 16 * i) * TPITCH + g];
-            c1[i] = lds[(r + 16 * i) * TPITCH + g + 32];
+            for (int i = 0; i < 16; ++i) c[i] = lds[(r + 16 * i) * TPITCH + g];
+            __syncthreads();
+            fwd_pass1_lds(c, twrow, gg);
+            wave_lds_fence();
+#pragma unroll
+            for (int q = 0; q < 16; ++q) exch[r * 17 + q] = gg[q];
+            wave_lds_fence();
+            cpx u[16];
+#pragma unroll
+            for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + r];
+            // only u[] is live now: start the next image's first row so HBM stays busy during the column pass
+            if (nxt < nimg) issue(v, nxt, 0);
+            dft16_first4<-1>(u, z);
         }
-        __syncthreads();
-        // the row registers are free again: start the next image's first rows before the column pass
-        if (nxt < nimg) { issue(va, nxt, 0); issue(vb, nxt, 1); }
-        group_forward<8>(c0, tw, exch, r, z0);
-        group_forward<8>(c1, tw, exch, r, z1);
         // lane order of the retained modes: element s*1024 + q*16 + r  <->  mode (p = r + 16 s, q)
-        float2* dst = spec + img * 4096 + g * 16 + r;
+        float2* dst = spec + img * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) { dst[1024 * s] = z0[s]; dst[1024 * s + 512] = z1[s]; }
+        for (int s = 0; s < 4; ++s) dst[(unsigned)tid + 1024u * s] = z[s];
     }
 }
 
@@ -238,7 +251,7 @@ hipError_t launch_fft2d_trunc_256(const float2* x, float2* spec, long nimg, hipS
     }
     // one persistent block per CU (the LDS tile allows exactly one resident block per CU)
     const long blocks = nimg < cu_count() ? nimg : cu_count();
-    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)blocks), dim3(512), LDS2D_FWD_BYTES, stream, x, spec,
+    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)blocks), dim3(1024), LDS2D_FWD_BYTES, stream, x, spec,
                        (int)nimg);
     return hipGetLastError();
 }
