@@ -72,7 +72,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
     cpx v[16];
     if (img < nimg) issue(v, img, 0);
     for (; img < nimg; img += gridDim.x) {
-        const long nxt = img + gridDim.x;
+        const long pre = img + gridDim.x < nimg ? img + gridDim.x : img;
         // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 64 it
         cpx T[4][4];
 #pragma unroll
@@ -80,7 +80,10 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
             cpx bb[16], gg[16];
             fft16_stage1<-1>(v, bb);
             // v is dead after the first radix-4 stage: its registers become the landing zone of the next row
+            // the last pass already fetches the next image's first row (for the final image: a harmless
+            // re-read of its own), so HBM stays busy through the redistribution and the column pass
             if (it + 1 < 4) issue(v, img, it + 1);
+            else issue(v, pre, 0);
             fwd_pass1_lds_finish(bb, twrow, gg);
             group_forward_finish<8>(gg, exch, r, T[it]);
         }
@@ -105,8 +108,6 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
             cpx u[16];
 #pragma unroll
             for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + r];
-            // only u[] is live now: start the next image's first row so HBM stays busy during the column pass
-            if (nxt < nimg) issue(v, nxt, 0);
             dft16_first4<-1>(u, z);
         }
         // lane order of the retained modes: element s*1024 + q*16 + r  <->  mode (p = r + 16 s, q)
@@ -168,8 +169,12 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
 constexpr int GEMM_WPITCH = 260;    // floats per k row of the W tile (256 + 4: spreads the k-major fill over banks)
-constexpr int GEMM_THREADS = 512;   // 8 waves, one 32-m strip each -> 256 m per block
+constexpr int GEMM_THREADS = 1024;  // 16 waves: 8 strips of 32 m x 2 halves of the 64-channel n tile
+constexpr int GEMM_MBLOCK = 256;    // m per block
 
+// Each wave owns a 32-m strip and one half (32 channels) of the n tile, i.e. two 32x32 accumulators. The four
+// waves that share a SIMD get descending issue priorities, so their matrix-core phases finish staggered and
+// the stores of one wave drain while the next wave still computes (otherwise all stores hit HBM at the end).
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
                                                                    const float2* __restrict__ W, float2* __restrict__ C,
                                                                    long Mtot, int N, int K, float2 alpha)
@@ -177,12 +182,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     // sW[k*260 + n'*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:  {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1
     __shared__ float sW[GEMM_KC * GEMM_WPITCH];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
-    const long m0 = ((long)blockIdx.x * (GEMM_THREADS / 64) + wave) * 32;
+    const int strip = wave >> 1, nh = wave & 1;
     const int n0 = blockIdx.y * 64;
+    switch (wave >> 2) {                      // waves w, w+4, w+8, w+12 share a SIMD
+    case 0: __builtin_amdgcn_s_setprio(3); break;
+    case 1: __builtin_amdgcn_s_setprio(2); break;
+    case 2: __builtin_amdgcn_s_setprio(1); break;
+    default: __builtin_amdgcn_s_setprio(0); break;
+    }
 
-    floatx16 acc[4];
+    floatx16 acc[2];
 #pragma unroll
-    for (int tI = 0; tI < 4; ++tI)
+    for (int tI = 0; tI < 2; ++tI)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[tI][e] = 0.f;
 
@@ -190,41 +201,55 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
         const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;
         // lane (col, half) feeds A[kc + kk + half][m0 + col] as {re, im}; all loads of the chunk are issued
         // before the W tile is built so their latency hides behind it
-        const float2* ap = A + (long)(kc + half) * Mtot + m0 + col;
+        // (scalar base per k pair + one 32-bit lane offset keeps the 32 addresses out of the vector registers)
+        const unsigned lane_off = (unsigned)(half * Mtot) + (unsigned)(strip * 32 + col);
         float2 bv[GEMM_KC / 2];
 #pragma unroll
-        for (int q = 0; q < GEMM_KC / 2; ++q)
-            bv[q] = (2 * q < kn) ? ap[(long)(2 * q) * Mtot] : make_float2(0.f, 0.f);
+        for (int q = 0; q < GEMM_KC / 2; ++q) {
+            const float2* base = A + (long)(kc + 2 * q) * Mtot + (long)blockIdx.x * GEMM_MBLOCK;
+            bv[q] = (2 * q < kn) ? base[lane_off] : make_float2(0.f, 0.f);
+        }
         __syncthreads();
-        for (int idx = tid; idx < GEMM_KC * 64; idx += GEMM_THREADS) {
+        // all W loads of the tile are issued before the first LDS store (one round trip)
+        constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
+        float2 wv[WPT];
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
             const int k = idx % GEMM_KC, n = idx / GEMM_KC;   // k fastest: coalesced reads of W[k + n*K]
-            float2 w = make_float2(0.f, 0.f);
-            if (k < kn) {
-                float2 w0 = W[(kc + k) + (long)(n0 + n) * K];
-                w = make_float2(w0.x * alpha.x - w0.y * alpha.y, w0.x * alpha.y + w0.y * alpha.x);
-            }
+            wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+            const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
             *reinterpret_cast<float4*>(&sW[k * GEMM_WPITCH + 4 * n]) = make_float4(w.x, -w.y, w.y, w.x);
         }
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < GEMM_KC / 2; ++q) {
 #pragma unroll
-            for (int tI = 0; tI < 4; ++tI) {
-                float2 a = *reinterpret_cast<const float2*>(&sW[(2 * q + half) * GEMM_WPITCH + (tI * 32 + col) * 2]);
+            for (int tI = 0; tI < 2; ++tI) {
+                float2 a = *reinterpret_cast<const float2*>(
+                    &sW[(2 * q + half) * GEMM_WPITCH + ((nh * 2 + tI) * 32 + col) * 2]);
                 acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bv[q].x, acc[tI], 0, 0, 0);
                 acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bv[q].y, acc[tI], 0, 0, 0);
             }
+            // keep the W-operand reads next to their matrix instructions (hoisting all 64 of them spills)
+            if ((q & 1) == 1) __builtin_amdgcn_sched_barrier(0);
         }
     }
     // D[row = 8 i + 4 half + jj*2 + c'][col]: row = 2 n_local + c'
 #pragma unroll
-    for (int tI = 0; tI < 4; ++tI)
+    for (int tI = 0; tI < 2; ++tI)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj) {
-                int n = n0 + tI * 16 + 4 * i + 2 * half + jj;
-                C[(long)n * Mtot + m0 + col] = make_float2(acc[tI][4 * i + 2 * jj], acc[tI][4 * i + 2 * jj + 1]);
+                float2* base = C + (long)(n0 + (nh * 2 + tI) * 16 + 4 * i + jj) * Mtot + (long)blockIdx.x * GEMM_MBLOCK;
+                base[(unsigned)(2 * half * Mtot) + (unsigned)(strip * 32 + col)] =
+                    make_float2(acc[tI][4 * i + 2 * jj], acc[tI][4 * i + 2 * jj + 1]);
             }
 }
 
@@ -272,8 +297,8 @@ hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipSt
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               hipStream_t stream)
 {
-    if (Mtot % 256 != 0 || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
-    dim3 grid((unsigned)(Mtot / 256), (unsigned)(N / 64), 1);
+    if (Mtot % GEMM_MBLOCK != 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(Mtot / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha);
     return hipGetLastError();
 }
