@@ -277,6 +277,17 @@ TFNO_DEV void inv_pass2(cpx (&e)[16], const cpx (&tw)[16], cpx (&y)[16])
 // lanes after. DS operations of a wave complete in issue order, so no hardware wait is needed
 // beyond what the compiler inserts for the data dependency; this only stops compiler reordering.
 #ifndef TFNO_HOST_CHECK
+// Streaming (non-temporal) global accesses for data touched exactly once.
+TFNO_DEV cpx load_streaming(const cpx* p)
+{
+    return make_float2(__builtin_nontemporal_load(&p->x), __builtin_nontemporal_load(&p->y));
+}
+TFNO_DEV void store_streaming(cpx* p, cpx v)
+{
+    __builtin_nontemporal_store(v.x, &p->x);
+    __builtin_nontemporal_store(v.y, &p->y);
+}
+
 TFNO_DEV void wave_lds_fence()
 {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -62,10 +62,12 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
     const int row0 = row_of(w, j, 0);
     // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
     const unsigned lane_off = (unsigned)(row0 * IMG + r);
+    // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
+    // next kernel re-reads, out of L2 / Infinity Cache
     auto issue = [&](cpx (&dst)[16], long img, int it) {
         const float2* base = x + (img * IMG + 64 * it) * (long)IMG;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = base[lane_off + 16u * i];
+        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[lane_off + 16u * i]);
     };
 
     long img = blockIdx.x;
@@ -150,9 +152,11 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __re
     for (int it = 0; it < 4; ++it) {
         cpx yv[16];
         group_backward<8>(cc[it], tw, exch, r, yv);
+        // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
+        // dirty lines from lingering in the Infinity Cache and being written back under the next kernel's reads
         float2* dst = y + (img * IMG + row_of(w, j, it)) * IMG + r;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[16 * i] = yv[i];
+        for (int i = 0; i < 16; ++i) store_streaming(&dst[16 * i], yv[i]);
     }
 }
 
