@@ -278,14 +278,16 @@ TFNO_DEV void inv_pass2(cpx (&e)[16], const cpx (&tw)[16], cpx (&y)[16])
 // beyond what the compiler inserts for the data dependency; this only stops compiler reordering.
 #ifndef TFNO_HOST_CHECK
 // Streaming (non-temporal) global accesses for data touched exactly once.
+typedef float tfno_v2f __attribute__((ext_vector_type(2)));
 TFNO_DEV cpx load_streaming(const cpx* p)
 {
-    return make_float2(__builtin_nontemporal_load(&p->x), __builtin_nontemporal_load(&p->y));
+    const tfno_v2f v = __builtin_nontemporal_load(reinterpret_cast<const tfno_v2f*>(p));
+    return make_float2(v.x, v.y);
 }
 TFNO_DEV void store_streaming(cpx* p, cpx v)
 {
-    __builtin_nontemporal_store(v.x, &p->x);
-    __builtin_nontemporal_store(v.y, &p->y);
+    tfno_v2f q = { v.x, v.y };
+    __builtin_nontemporal_store(q, reinterpret_cast<tfno_v2f*>(p));
 }
 
 TFNO_DEV void wave_lds_fence()

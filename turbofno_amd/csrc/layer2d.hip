@@ -119,44 +119,64 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
     }
 }
 
-__global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __restrict__ spec, float2* __restrict__ y)
+// Backward image kernel, mirror of the forward one: persistent blocks, 16 waves per CU, twiddles in LDS.
+// The 32 KiB spectrum of the next image is fetched (4 registers per lane) while the current image's rows
+// are being transformed and stored, so a CU never waits for its input between images.
+__global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
+                                                              int nimg)
 {
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
-    const long img = blockIdx.x;
     float2* exch = lds + g * EXCH256;
+    float2* twtab = lds + LDS2D_ELEMS;
+    fill_lds_twiddles<8>(twtab, tid, 1024);
+    const float2* twrow = twtab + r * kTwLdsPitch;
+    __syncthreads();
 
-    cpx tw[16];
-    load_lane_twiddles<8>(r, tw);
+    const int row0 = row_of(w, j, 0);
+    const unsigned lane_off = (unsigned)(row0 * IMG + r);
 
-    // pass 1: columns (p -> x) of column q = g
-    {
-        const float2* src = spec + img * 4096 + tid;
-        cpx c[4], u[16];
+    long img = blockIdx.x;
+    cpx c[4];
+    if (img < nimg) {
+        const float2* src = spec + img * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) c[s] = src[1024 * s];
-        group_backward<8>(c, tw, exch, r, u);
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 16; ++i) lds[(r + 16 * i) * TPITCH + g] = u[i];
+        for (int s = 0; s < 4; ++s) c[s] = src[(unsigned)tid + 1024u * s];
     }
-    __syncthreads();
-    cpx cc[4][4];
+    for (; img < nimg; img += gridDim.x) {
+        const long pre = img + gridDim.x < nimg ? img + gridDim.x : img;
+        // pass 1: columns (p -> x) of column q = g
+        {
+            cpx u[16];
+            group_backward256_lds(c, twrow, exch, r, u);
+            __syncthreads();
 #pragma unroll
-    for (int it = 0; it < 4; ++it)
+            for (int i = 0; i < 16; ++i) lds[(r + 16 * i) * TPITCH + g] = u[i];
+        }
+        // next image's spectrum (for the last image: a harmless re-read of its own)
+        {
+            const float2* src = spec + pre * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) cc[it][s] = lds[row_of(w, j, it) * TPITCH + r + 16 * s];
-    __syncthreads();
-    // pass 2: rows (q -> y), coalesced 2 KiB row stores
+            for (int s = 0; s < 4; ++s) c[s] = src[(unsigned)tid + 1024u * s];
+        }
+        __syncthreads();
+        cpx cc[4][4];
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        cpx yv[16];
-        group_backward<8>(cc[it], tw, exch, r, yv);
+        for (int it = 0; it < 4; ++it)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) cc[it][s] = lds[(row0 + 64 * it) * TPITCH + r + 16 * s];
+        __syncthreads();
+        // pass 2: rows (q -> y), coalesced 2 KiB row stores.
         // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
         // dirty lines from lingering in the Infinity Cache and being written back under the next kernel's reads
-        float2* dst = y + (img * IMG + row_of(w, j, it)) * IMG + r;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) store_streaming(&dst[16 * i], yv[i]);
+        for (int it = 0; it < 4; ++it) {
+            cpx yv[16];
+            group_backward256_lds(cc[it], twrow, exch, r, yv);
+            float2* dst = y + (img * IMG + 64 * it) * (long)IMG;   // uniform base + lane offset + immediates
+#pragma unroll
+            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + 16 * i, yv[i]);
+        }
     }
 }
 
@@ -290,11 +310,13 @@ hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipSt
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ifft2d_pad_256_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_FWD_BYTES);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(ifft2d_pad_256_kernel, dim3((unsigned)nimg), dim3(1024), LDS2D_BYTES, stream, spec, y);
+    const long blocks = nimg < cu_count() ? nimg : cu_count();
+    hipLaunchKernelGGL(ifft2d_pad_256_kernel, dim3((unsigned)blocks), dim3(1024), LDS2D_FWD_BYTES, stream, spec, y,
+                       (int)nimg);
     return hipGetLastError();
 }
 
