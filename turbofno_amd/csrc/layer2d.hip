@@ -186,27 +186,29 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __re
 // Same contraction as the reference's cgemm / the GEMM phase of its fused kernel
 // (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4-205, operand layout lda=M, ldb=K, ldc=M),
 // expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition) on
-// v_mfma_f32_32x32x2_f32: rows = (n, re/im), cols = 32 consecutive m, contraction = (k, re/im).
-// One wave owns a 32-m strip and a 64-channel n tile (4 accumulators of 32x32).
+// v_mfma_f32_16x16x4_f32: rows = (n, re/im), cols = 16 consecutive m, contraction = 4 channels x re|im.
+// A block is 16 waves; wave w owns the 16-m strip w and the whole 64-channel n tile (8 accumulators of
+// 16x16), so every element of A is loaded exactly once. One float2 load per lane feeds two matrix
+// instructions per n tile (real parts, then imaginary parts). The K loop runs in quarters whose loads are
+// issued one quarter ahead; the four waves of a SIMD get descending priorities so that they finish
+// staggered and the stores of one drain under the matrix work of the others.
 // ---------------------------------------------------------------------------------------------
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
-constexpr int GEMM_WPITCH = 260;    // floats per k row of the W tile (256 + 4: spreads the k-major fill over banks)
-constexpr int GEMM_THREADS = 1024;  // 16 waves: 8 strips of 32 m x 2 halves of the 64-channel n tile
+constexpr int GEMM_WGROUP = 1024;   // floats per group of 4 channels in the W tile: [(k&3)>>1][n' (128)][k&1][c]
+constexpr int GEMM_THREADS = 1024;  // 16 waves x 16 m
 constexpr int GEMM_MBLOCK = 256;    // m per block
 
-// Each wave owns a 32-m strip and one half (32 channels) of the n tile, i.e. two 32x32 accumulators. The four
-// waves that share a SIMD get descending issue priorities, so their matrix-core phases finish staggered and
-// the stores of one wave drain while the next wave still computes (otherwise all stores hit HBM at the end).
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
                                                                    const float2* __restrict__ W, float2* __restrict__ C,
                                                                    long Mtot, int N, int K, float2 alpha)
 {
-    // sW[k*260 + n'*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:  {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1
-    __shared__ float sW[GEMM_KC * GEMM_WPITCH];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
-    const int strip = wave >> 1, nh = wave & 1;
+    // sW[(k/4)*1024 + ((k&3)>>1)*512 + n'*4 + (k&1)*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:
+    // {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1. In one operand read (16 n' x 4 channels) lanes 0-31 cover 256
+    // contiguous bytes in lane order pairs and lanes 32-63 the next 256: no bank conflicts.
+    __shared__ float sW[(GEMM_KC / 4) * GEMM_WGROUP];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.y * 64;
     switch (wave >> 2) {                      // waves w, w+4, w+8, w+12 share a SIMD
     case 0: __builtin_amdgcn_s_setprio(3); break;
@@ -215,66 +217,69 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     default: __builtin_amdgcn_s_setprio(0); break;
     }
 
-    floatx16 acc[2];
+    floatx4 acc[8];
 #pragma unroll
-    for (int tI = 0; tI < 2; ++tI)
+    for (int t = 0; t < 8; ++t) acc[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
+
+    // scalar base per k group + one 32-bit lane offset keeps the addresses out of the vector registers
+    const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
+    const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
+    auto load_quarter = [&](float2 (&dst)[4], int kc, int kn, int quarter) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[tI][e] = 0.f;
+        for (int jj = 0; jj < 4; ++jj) {
+            const int k4 = 16 * quarter + 4 * jj;            // lane reads channel kc + k4 + kq
+            dst[jj] = (k4 < kn) ? (blk + (long)(kc + k4) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+        }
+    };
 
     for (int kc = 0; kc < K; kc += GEMM_KC) {
-        const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;
-        // lane (col, half) feeds A[kc + kk + half][m0 + col] as {re, im}; all loads of the chunk are issued
-        // before the W tile is built so their latency hides behind it
-        // (scalar base per k pair + one 32-bit lane offset keeps the 32 addresses out of the vector registers)
-        const unsigned lane_off = (unsigned)(half * Mtot) + (unsigned)(strip * 32 + col);
-        float2 bv[GEMM_KC / 2];
-#pragma unroll
-        for (int q = 0; q < GEMM_KC / 2; ++q) {
-            const float2* base = A + (long)(kc + 2 * q) * Mtot + (long)blockIdx.x * GEMM_MBLOCK;
-            bv[q] = (2 * q < kn) ? base[lane_off] : make_float2(0.f, 0.f);
-        }
+        const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;   // multiple of 8 (caller contract)
+        float2 bv[2][4];
+        load_quarter(bv[0], kc, kn, 0);
         __syncthreads();
-        // all W loads of the tile are issued before the first LDS store (one round trip)
+        // W tile: lanes run along n so each LDS store is a conflict-free 16 B; W itself is tiny and cached
         constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
         float2 wv[WPT];
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % GEMM_KC, n = idx / GEMM_KC;   // k fastest: coalesced reads of W[k + n*K]
+            const int n = idx % 64, k = idx / 64;
             wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+            const int n = idx % 64, k = idx / 64;
             const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
-            *reinterpret_cast<float4*>(&sW[k * GEMM_WPITCH + 4 * n]) = make_float4(w.x, -w.y, w.y, w.x);
+            float* dstw = &sW[(k >> 2) * GEMM_WGROUP + ((k & 3) >> 1) * 512 + (2 * n) * 4 + (k & 1) * 2];
+            *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
+            *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
         }
         __syncthreads();
 #pragma unroll
-        for (int q = 0; q < GEMM_KC / 2; ++q) {
+        for (int quarter = 0; quarter < 4; ++quarter) {
+            if (quarter + 1 < 4) load_quarter(bv[(quarter + 1) & 1], kc, kn, quarter + 1);
 #pragma unroll
-            for (int tI = 0; tI < 2; ++tI) {
-                float2 a = *reinterpret_cast<const float2*>(
-                    &sW[(2 * q + half) * GEMM_WPITCH + ((nh * 2 + tI) * 32 + col) * 2]);
-                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bv[q].x, acc[tI], 0, 0, 0);
-                acc[tI] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bv[q].y, acc[tI], 0, 0, 0);
+            for (int jj = 0; jj < 4; ++jj) {
+                const int kg = 4 * quarter + jj;             // channel group; this lane's channel is 4 kg + kq
+                const float2 b = bv[quarter & 1][jj];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float2 a = *reinterpret_cast<const float2*>(&sW[kg * GEMM_WGROUP + (kq >> 1) * 512 + (t * 16 + col) * 4 + (kq & 1) * 2]);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[t], 0, 0, 0);
+                }
             }
-            // keep the W-operand reads next to their matrix instructions (hoisting all 64 of them spills)
-            if ((q & 1) == 1) __builtin_amdgcn_sched_barrier(0);
         }
     }
-    // D[row = 8 i + 4 half + jj*2 + c'][col]: row = 2 n_local + c'
+    // D[row = 4 kq + v][col]: row n' = 16 t + 4 kq + v = 2 n_local + c'  ->  n_local = 8 t + 2 kq + (v >> 1)
+    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
+    const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
 #pragma unroll
-    for (int tI = 0; tI < 2; ++tI)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                float2* base = C + (long)(n0 + (nh * 2 + tI) * 16 + 4 * i + jj) * Mtot + (long)blockIdx.x * GEMM_MBLOCK;
-                base[(unsigned)(2 * half * Mtot) + (unsigned)(strip * 32 + col)] =
-                    make_float2(acc[tI][4 * i + 2 * jj], acc[tI][4 * i + 2 * jj + 1]);
-            }
+    for (int t = 0; t < 8; ++t) {
+        (cblk + (long)(n0 + 8 * t) * Mtot)[out_off] = make_float2(acc[t][0], acc[t][1]);
+        (cblk + (long)(n0 + 8 * t + 1) * Mtot)[out_off] = make_float2(acc[t][2], acc[t][3]);
+    }
 }
 
 static int cu_count()
@@ -323,7 +328,7 @@ hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipSt
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               hipStream_t stream)
 {
-    if (Mtot % GEMM_MBLOCK != 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 2 != 0) return hipErrorInvalidValue;
+    if (Mtot % GEMM_MBLOCK != 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)(Mtot / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha);
     return hipGetLastError();
