@@ -26,6 +26,8 @@ def main():
     ap.add_argument("--algo", type=int, default=0, help="0 auto, 1 three-kernel pipeline, 2 whole-image")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-comparators", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 512 MiB device copy (calibrates FETCH_SIZE/WRITE_SIZE under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets ONE GPU (the layer shards over the batch with no exchange; "
@@ -48,6 +50,11 @@ def main():
 
     def step():
         tf.layer_2d(x, W, y=y, alpha=1.0, workspace=ws, algo=args.algo)
+
+    if args.copy_probe:
+        # plain copy of known size: y[:512 MiB] <- x; the counters of this dispatch give the KiB-per-unit scale
+        y.view(-1)[: x.numel()].copy_(x.view(-1))
+        torch.cuda.synchronize()
 
     for _ in range(args.warmup):
         step()
@@ -98,6 +105,16 @@ def main():
                     "algorithmic_bytes_per_launch": layer_bytes}
 
     layer_gbs = layer_bytes / (ms * 1e-3) / 1e9
+
+    # HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc summary (FETCH_SIZE and
+    # WRITE_SIZE scaled by a plain copy of known size); null when no summary is present for this workload
+    try:
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "layer2d_traffic.json")) as f:
+            tr = json.load(f)
+        if roofline and tr.get("workload") == "bs=%d 256x256 K=%d N=%d" % (bs, K, N):
+            roofline["traffic"] = tr["kernels"].get(roofline["kernel"], {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError, KeyError):
+        pass
 
     # ---- comparators on the same inputs (informational) ------------------------------------------
     comparators = {}

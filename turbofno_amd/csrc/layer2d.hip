@@ -64,17 +64,21 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
     const unsigned lane_off = (unsigned)(row0 * IMG + r);
     // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
     // next kernel re-reads, out of L2 / Infinity Cache
-    auto issue = [&](cpx (&dst)[16], long img, int it) {
+    auto issue = [&](cpx (&dst)[16], long img, int it, unsigned off) {
         const float2* base = x + (img * IMG + 64 * it) * (long)IMG;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[lane_off + 16u * i]);
+        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + 16u * i]);
     };
 
     long img = blockIdx.x;
     cpx v[16];
-    if (img < nimg) issue(v, img, 0);
+    if (img < nimg) issue(v, img, 0, lane_off);
     for (; img < nimg; img += gridDim.x) {
-        const long pre = img + gridDim.x < nimg ? img + gridDim.x : img;
+        // look-ahead target: the next image's first rows; after the last image every lane group re-reads the
+        // same 2 KiB (row 0 of image 0, cache resident) so the loop stays branch free at no HBM cost
+        const bool more = img + gridDim.x < nimg;
+        const long pre = more ? img + gridDim.x : 0;
+        const unsigned pre_off = more ? lane_off : (unsigned)r;
         // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 64 it
         cpx T[4][4];
 #pragma unroll
@@ -84,8 +88,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
             // v is dead after the first radix-4 stage: its registers become the landing zone of the next row
             // the last pass already fetches the next image's first row (for the final image: a harmless
             // re-read of its own), so HBM stays busy through the redistribution and the column pass
-            if (it + 1 < 4) issue(v, img, it + 1);
-            else issue(v, pre, 0);
+            if (it + 1 < 4) issue(v, img, it + 1, lane_off);
+            else issue(v, pre, 0, pre_off);
             fwd_pass1_lds_finish(bb, twrow, gg);
             group_forward_finish<8>(gg, exch, r, T[it]);
         }
