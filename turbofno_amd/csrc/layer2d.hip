@@ -117,9 +117,10 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
             dft16_first4<-1>(u, z);
         }
         // lane order of the retained modes: element s*1024 + q*16 + r  <->  mode (p = r + 16 s, q)
+        // written through as it is produced, so the end-of-kernel cache write-back has nothing left to flush
         float2* dst = spec + img * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) dst[(unsigned)tid + 1024u * s] = z[s];
+        for (int s = 0; s < 4; ++s) store_streaming(dst + tid + 1024 * s, z[s]);
     }
 }
 
@@ -241,19 +242,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
         float2 bv[2][4];
         load_quarter(bv[0], kc, kn, 0);
         __syncthreads();
-        // W tile: lanes run along n so each LDS store is a conflict-free 16 B; W itself is tiny and cached
+        // W tile: lanes run along k, the contiguous direction of W[k + n*K], so a wave reads 512 contiguous bytes
+        // (the LDS stores then collide on banks, but there are only eight of them per lane)
         constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
         float2 wv[WPT];
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * GEMM_THREADS;
-            const int n = idx % 64, k = idx / 64;
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
             wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * GEMM_THREADS;
-            const int n = idx % 64, k = idx / 64;
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
             const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
             float* dstw = &sW[(k >> 2) * GEMM_WGROUP + ((k & 3) >> 1) * 512 + (2 * n) * 4 + (k & 1) * 2];
             *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
@@ -281,8 +283,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        (cblk + (long)(n0 + 8 * t) * Mtot)[out_off] = make_float2(acc[t][0], acc[t][1]);
-        (cblk + (long)(n0 + 8 * t + 1) * Mtot)[out_off] = make_float2(acc[t][2], acc[t][3]);
+        store_streaming(cblk + (long)(n0 + 8 * t) * Mtot + out_off, make_float2(acc[t][0], acc[t][1]));
+        store_streaming(cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off, make_float2(acc[t][2], acc[t][3]));
     }
 }
 
