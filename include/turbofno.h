@@ -39,7 +39,7 @@ extern "C" {
 /* algorithms of turbofno_layer_2d */
 #define TURBOFNO_2D_AUTO          0
 #define TURBOFNO_2D_THREE_KERNEL  1  /* X transform, fused Y stage, X inverse: the reference's structure */
-#define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM (DX = DY = 256)          */
+#define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM (default)                */
 
 /*
  * Fused 1D layer kernel. Replaces the table entries fused_fft_cgemm_ifft[log2(DY)-7]
@@ -80,7 +80,7 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:133-172). The reference keeps its
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
- * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE when DX = DY = 256, else THREE_KERNEL.
+ * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE.
  */
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo);
 int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,
@@ -92,13 +92,13 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
  *   turbofno_fft2d_trunc : x[nimg][DX][DY] -> spec[nimg][4096]  truncated 2D forward transform per image
  *   turbofno_ifft2d_pad  : spec[nimg][4096] -> y[nimg][DX][DY]  zero-padded 2D backward transform per image
  * The 4096 retained modes of an image are stored in an order private to these two kernels (element
- * s*1024 + q*16 + r holds mode (p = r + 16 s, q)); a GEMM over the channel dimension does not care.
- * Requires DX = DY = 256.
+ * mm*(4*DX) + q*(DX/16) + t holds mode (p = t + (DX/16)*mm, q)); a GEMM over the channel dimension does
+ * not care. Requires DX, DY in {128, 256}.
  *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] (column major, lda = M, ldb = K,
  *   ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
  *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:182-200) for beta = 0,
- *   the only value with which the fused variant D uses the product. Requires M % 256 == 0, N % 64 == 0,
- *   K % 8 == 0.
+ *   the only value with which the fused variant D uses the product. Requires M % 256 == 0, M < 2^27,
+ *   N % 64 == 0, K % 8 == 0.
  */
 int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream);
 int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, void* stream);

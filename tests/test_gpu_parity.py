@@ -68,6 +68,10 @@ def test_stride_stages(DX, DY, nsig, tol):
     (1, 256, 256, 16, 64, 2),
     (2, 256, 256, 8, 128, 2),
     (1, 256, 256, 72, 64, 2),        # K crosses the 64-channel W chunk of the matrix-core GEMM
+    (1, 128, 128, 16, 64, 2),        # whole-image kernels for the other three built shapes
+    (3, 128, 256, 8, 64, 2),
+    (2, 256, 128, 24, 128, 2),
+    (5, 128, 128, 8, 64, 0),         # auto, more images than one pass of the persistent grid would need
 ])
 def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     print("case layer_2d", bs, DX, DY, K, N, algo, flush=True)

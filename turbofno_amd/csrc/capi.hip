@@ -45,7 +45,11 @@ int check_gemm_dims(long M, int N, int K)
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-int pick_algo(int DX, int DY, int algo) { return algo != TURBOFNO_2D_AUTO ? algo : (DX == 256 && DY == 256 ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL); }
+int pick_algo(int DX, int DY, int algo)
+{
+    (void)DX; (void)DY;   // every built shape has a whole-image kernel
+    return algo != TURBOFNO_2D_AUTO ? algo : TURBOFNO_2D_WHOLE_IMAGE;
+}
 
 }  // namespace
 
@@ -105,16 +109,20 @@ int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, v
 {
     if (!x || !spec) return fail(TURBOFNO_ERR_INVALID_ARG, "x and spec must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
-    if (DX != 256 || DY != 256) return fail(TURBOFNO_ERR_UNSUPPORTED, "whole-image transforms are built for DX = DY = 256 only");
-    return hip_status(tfno::launch_fft2d_trunc_256((const float2*)x, (float2*)spec, nimg, (hipStream_t)stream), "fft2d_trunc launch");
+    const int logDX = log2_exact(DX), logDY = log2_exact(DY);
+    if (!length_built(logDX) || !length_built(logDY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
+    return hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, (float2*)spec, nimg, (hipStream_t)stream), "fft2d_trunc launch");
 }
 
 int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, void* stream)
 {
     if (!spec || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "spec and y must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
-    if (DX != 256 || DY != 256) return fail(TURBOFNO_ERR_UNSUPPORTED, "whole-image transforms are built for DX = DY = 256 only");
-    return hip_status(tfno::launch_ifft2d_pad_256((const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
+    const int logDX = log2_exact(DX), logDY = log2_exact(DY);
+    if (!length_built(logDX) || !length_built(logDY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
+    return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, (const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
 }
 
 int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im, void* stream)
@@ -122,6 +130,7 @@ int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, 
     if (!A || !B || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "A, B and C must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
     if (M % 256) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld is not a multiple of the 256-row block tile", M);
+    if (M >= (1L << 27)) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld exceeds the 2^27 rows the 32-bit lane offsets cover", M);
     return hip_status(tfno::launch_cgemm_modes((const float2*)A, (const float2*)B, (float2*)C, M, N, K,
                                                make_float2(alpha_re, alpha_im), (hipStream_t)stream), "cgemm launch");
 }
@@ -147,8 +156,6 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE)
         return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
     const int a = pick_algo(DX, DY, algo);
-    if (a == TURBOFNO_2D_WHOLE_IMAGE && !(DX == 256 && DY == 256))
-        return fail(TURBOFNO_ERR_UNSUPPORTED, "the whole-image algorithm is built for DX = DY = 256 only");
     const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
     if (!workspace || workspace_bytes < need)
         return fail(TURBOFNO_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need, workspace ? workspace_bytes : (size_t)0);
@@ -159,9 +166,9 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     if (a == TURBOFNO_2D_WHOLE_IMAGE) {
         float2* spec = (float2*)ws;
         float2* cspec = (float2*)(ws + align256((size_t)K * bs * 4096 * sizeof(float2)));
-        if (int rc = hip_status(tfno::launch_fft2d_trunc_256((const float2*)x, spec, (long)K * bs, st), "fft2d_trunc launch")) return rc;
+        if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, (long)K * bs, st), "fft2d_trunc launch")) return rc;
         if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, st), "cgemm_modes launch")) return rc;
-        return hip_status(tfno::launch_ifft2d_pad_256(cspec, (float2*)y, (long)N * bs, st), "ifft2d_pad launch");
+        return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, (long)N * bs, st), "ifft2d_pad launch");
     }
     float2* t1 = (float2*)ws;
     float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));

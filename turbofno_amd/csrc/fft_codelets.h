@@ -203,7 +203,7 @@ constexpr int kTwLdsSize = 16 * kTwLdsPitch;   // complex elements
 #ifndef TFNO_HOST_CHECK
 template <int LOGD> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
 {
-    for (int e = tid; e < 256; e += nthreads) {
+    for (int e = tid; e < 16 * ((1 << LOGD) / 16); e += nthreads) {
         const int t = e >> 4, r = e & 15;
         tab[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
     }

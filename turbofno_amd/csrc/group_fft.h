@@ -80,14 +80,27 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
     inv_pass2(e, tw, y);
 }
 
-// zero-padded backward transform (L = 16) whose last pass takes its twiddles from an LDS table row.
-TFNO_DEV void group_backward256_lds(const cpx (&c)[4], const cpx* twrow, cpx* exch, int t, cpx (&y)[16])
+// zero-padded backward transform whose last pass takes its twiddles from an LDS table row
+// (twrow = table + t * kTwLdsPitch). Lane t holds modes m = t + L*mm in c[]; returns samples t + L*i in y[].
+template <int LOGD>
+TFNO_DEV void group_backward_lds(const cpx (&c)[Geo1D<LOGD>::MM], const cpx* twrow, cpx* exch, int t, cpx (&y)[16])
 {
+    constexpr int L = Geo1D<LOGD>::L;
     wave_lds_fence();
-    cpx h[16];
-    dft16_pad4<+1>(c, h);
+    if constexpr (L == 16) {
+        cpx h[16];
+        dft16_pad4<+1>(c, h);
 #pragma unroll
-    for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+        for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+    } else {
+        cpx c0[4], c1[4], h0[8], h1[8];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { c0[s] = c[2 * s]; c1[s] = c[2 * s + 1]; }
+        dft8_pad4<+1>(c0, h0);
+        dft8_pad4<+1>(c1, h1);
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) { exch[tt * 17 + t] = h0[tt]; exch[tt * 17 + t + 8] = h1[tt]; }
+    }
     wave_lds_fence();
     cpx e[16];
 #pragma unroll

@@ -12,10 +12,10 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
 hipError_t launch_fft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream);
 hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream);
 
-// Whole-image 2D path (DX = DY = 256): truncated 2D forward transform per image, mode-space CGEMM
+// Whole-image 2D path (DX, DY in {128, 256}): truncated 2D forward transform per image, mode-space CGEMM
 // on the matrix cores, zero-padded 2D backward transform per image.
-hipError_t launch_fft2d_trunc_256(const float2* x, float2* spec, long nimg, hipStream_t stream);
-hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipStream_t stream);
+hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, long nimg, hipStream_t stream);
+hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, long nimg, hipStream_t stream);
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               hipStream_t stream);
 

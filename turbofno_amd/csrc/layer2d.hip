@@ -1,73 +1,90 @@
-// Whole-image 2D spectral layer for 256 x 256 grids (the MI355X-first path of the 2D layer).
+// Whole-image 2D spectral layer (the MI355X-first path of the 2D layer), DX, DY in {128, 256}.
 //
 // The reference's "fully fused" 2D variant is three kernels with two HBM round trips of
 // half-truncated intermediates (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:150-172:
 // X transform -> t1[K*bs][64][DY], fused Y stage, t2[N*bs][64][DY] -> X inverse). Here one 1024-thread
-// block owns a whole 256 x 256 image, so only fully truncated 64 x 64 spectra (1/16 of the image)
-// ever leave the CU:
+// block owns a whole DX x DY image, so only fully truncated 64 x 64 spectra ever leave the CU:
 //
-//   fft2d_trunc_256   image (k,b): 256 row FFTs along Y (coalesced 2 KiB rows, 64 modes kept, held in
-//                     registers), redistribution through LDS, 64 column FFTs along X (64 modes kept)
-//                     -> spec[k][b][4096]                                       reads 512 KiB, writes 32 KiB
-//   cgemm_modes       C[n][b][m] = alpha * sum_k W[k][n] spec[k][b][m] on the fp32 matrix cores
-//   ifft2d_pad_256    exact mirror -> y[n][b][256][256]                         reads 32 KiB, writes 512 KiB
+//   fft2d_trunc    image (k,b): DX row FFTs along Y (coalesced rows, 64 modes kept, held in registers),
+//                  redistribution through LDS, 64 column FFTs along X (64 modes kept)
+//                  -> spec[k][b][4096]                          reads 8 DX DY bytes, writes 32 KiB
+//   cgemm_modes    C[n][b][m] = alpha * sum_k W[k][n] spec[k][b][m] on the fp32 matrix cores
+//   ifft2d_pad     exact mirror -> y[n][b][DX][DY]              reads 32 KiB, writes 8 DX DY bytes
 //
 // so x is read once and y written once; padded / discarded modes are never touched in memory.
-// The 4096 modes of an image are stored in "lane order": element s*1024 + q*16 + r holds mode
-// (p = r + 16 s, q). That order is private to these three kernels (producer and consumer lanes
-// coincide, every access is a contiguous 512 B per wavefront) and the GEMM is oblivious to it.
+// The 4096 modes of an image are stored in "lane order": element mm*(64 LX) + q*LX + t holds mode
+// (p = t + LX mm, q), LX = DX/16. That order is private to the two image kernels (producer and consumer
+// lanes coincide, every access is contiguous per wavefront) and the GEMM is oblivious to it.
 #include "group_fft.h"
 #include "kernels.h"
 
 namespace tfno {
 
 namespace {
-constexpr int IMG = 256;
-constexpr int TPITCH = 66;                       // row pitch (complex) of the 256 x 64 redistribution tile
-constexpr int EXCH256 = 16 * 17;                 // exchange region of one 16-lane group
-constexpr int LDS2D_ELEMS = 64 * EXCH256 > IMG * TPITCH ? 64 * EXCH256 : IMG * TPITCH;   // exchange regions alias the tile
-constexpr size_t LDS2D_BYTES = sizeof(float2) * (size_t)LDS2D_ELEMS;
-constexpr size_t LDS2D_FWD_BYTES = sizeof(float2) * (size_t)(LDS2D_ELEMS + kTwLdsSize);
+constexpr int TPITCH = 66;                       // row pitch (complex) of the DX x 64 redistribution tile
+constexpr int EXCH_ELEMS = 1024 * 17;            // exchange regions of all lane groups of a 1024-thread block
 
-// Row handled by 16-lane group j of wave w in pass `it` (64 groups per block): groups 0/1 of a wave are
-// 8 rows apart so the two groups that share an LDS cycle hit disjoint banks in the pitch-66 tile.
-__device__ __forceinline__ int row_of(int w, int j, int it)
+// Geometry of the whole-image kernels for a DX x DY image (DX rows of DY contiguous samples).
+template <int LOGX, int LOGY> struct Geo2D {
+    static constexpr int DX = 1 << LOGX, DY = 1 << LOGY;
+    static constexpr int LX = DX / 16, LY = DY / 16;          // lanes per column / per row transform
+    static constexpr int GY = 1024 / LY;                      // rows transformed concurrently
+    static constexpr int ITY = DX / GY;                       // row passes per image
+    static constexpr int MMY = 64 / LY, MMX = 64 / LX;        // modes per lane after a row / column transform
+    static constexpr int COLT = 64 * LX;                      // threads that take part in the column pass
+    static constexpr int TILE = DX * TPITCH;
+    static constexpr int LDS_MAIN = EXCH_ELEMS > TILE ? EXCH_ELEMS : TILE;   // exchange regions alias the tile
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(LDS_MAIN + 2 * kTwLdsSize);
+    static_assert(ITY >= 1 && COLT <= 1024, "unsupported image shape");
+};
+
+// Row (within one pass of GY rows) handled by lane group g. The 32/LY groups that share an LDS cycle (one half
+// wavefront) get rows LY/2 apart, so that their pitch-66 tile accesses fall on disjoint banks.
+template <int LY> __device__ __forceinline__ int row_in_pass(int g)
 {
-    return 64 * it + ((w & 7) | ((j & 1) << 3) | ((j >> 1) << 4) | ((w >> 3) << 5));
-}
-// same for a 512-thread block (32 groups, 8 passes)
-__device__ __forceinline__ int row_of32(int w, int j, int it)
-{
-    return 32 * it + (w | ((j & 1) << 3) | ((j >> 1) << 4));
+    constexpr int GH = 32 / LY, HS = LY / 2;     // groups per half wavefront, row spacing between them
+    const int jh = g % GH, rest = g / GH;
+    return jh * HS + (rest % HS) + (rest / HS) * 16;
 }
 }  // namespace
 
-// Forward image kernel. 1024 threads = 64 lane groups = 16 waves per CU (4 per SIMD: the arithmetic
-// is issue bound, so full occupancy matters more than registers). A block is persistent over images
-// (img = blockIdx.x, += gridDim.x). Each group keeps ONE row in flight: the loads of its next row are
-// issued as soon as the first pass has consumed the row registers, so they travel while the exchange
-// and the second pass run, across the column pass and across image boundaries. Inter-pass twiddles
-// live in LDS to keep the kernel at 128 VGPRs.
-__global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
-                                                               int nimg)
+// Forward image kernel: truncated 2D transform of one DX x DY image per block iteration.
+// 1024 threads = 16 waves per CU (4 per SIMD: the arithmetic is issue bound, so full occupancy matters more
+// than registers). A block is persistent over images (img = blockIdx.x, += gridDim.x). Pass 1 transforms the
+// rows (along Y) with LY-lane groups and keeps the 64 retained modes of every row in registers; a pitch-66
+// LDS tile redistributes them; pass 2 transforms the 64 columns (along X) with LX-lane groups.
+// Each group keeps ONE row in flight: the loads of its next row are issued as soon as the first radix-4
+// stage has consumed the row registers, so they travel while the rest of the transform runs, across the
+// column pass and across image boundaries. Inter-pass twiddles live in LDS to stay within 128 VGPRs.
+template <int LOGX, int LOGY>
+__global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
+                                                           int nimg)
 {
+    using G = Geo2D<LOGX, LOGY>;
+    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, GY = G::GY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
-    float2* exch = lds + g * EXCH256;
-    float2* twtab = lds + LDS2D_ELEMS;                 // after the exchange regions / tile
-    fill_lds_twiddles<8>(twtab, tid, 1024);
-    const float2* twrow = twtab + r * kTwLdsPitch;
+    const int tid = threadIdx.x;
+    const int gy = tid / LY, ty = tid % LY;            // row pass: group and lane
+    const int gx = tid / LX, tx = tid % LX;            // column pass: group (= column q) and lane
+    float2* exch_y = lds + gy * (LY * 17);
+    float2* exch_x = lds + gx * (LX * 17);
+    float2* twtab_y = lds + G::LDS_MAIN;               // after the exchange regions / tile
+    float2* twtab_x = twtab_y + kTwLdsSize;
+    fill_lds_twiddles<LOGY>(twtab_y, tid, 1024);
+    fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
+    const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
+    const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
     __syncthreads();
 
-    const int row0 = row_of(w, j, 0);
+    const int row0 = row_in_pass<LY>(gy);
     // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
-    const unsigned lane_off = (unsigned)(row0 * IMG + r);
+    const unsigned lane_off = (unsigned)(row0 * DY + ty);
     // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
     // next kernel re-reads, out of L2 / Infinity Cache
     auto issue = [&](cpx (&dst)[16], long img, int it, unsigned off) {
-        const float2* base = x + (img * IMG + 64 * it) * (long)IMG;
+        const float2* base = x + (img * DX + GY * it) * (long)DY;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + 16u * i]);
+        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + (unsigned)(LY * i)]);
     };
 
     long img = blockIdx.x;
@@ -75,112 +92,115 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_256_kernel(const float2* __r
     if (img < nimg) issue(v, img, 0, lane_off);
     for (; img < nimg; img += gridDim.x) {
         // look-ahead target: the next image's first rows; after the last image every lane group re-reads the
-        // same 2 KiB (row 0 of image 0, cache resident) so the loop stays branch free at no HBM cost
+        // same row (row 0 of image 0, cache resident) so the loop stays branch free at no HBM cost
         const bool more = img + gridDim.x < nimg;
         const long pre = more ? img + gridDim.x : 0;
-        const unsigned pre_off = more ? lane_off : (unsigned)r;
-        // pass 1: rows (along Y). T[it][s] = mode q = r + 16 s of row row0 + 64 it
-        cpx T[4][4];
+        const unsigned pre_off = more ? lane_off : (unsigned)ty;
+        // pass 1: rows (along Y). T[it][mm] = mode q = ty + LY mm of row row0 + GY it
+        cpx T[ITY][MMY];
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
+        for (int it = 0; it < ITY; ++it) {
             cpx bb[16], gg[16];
             fft16_stage1<-1>(v, bb);
-            // v is dead after the first radix-4 stage: its registers become the landing zone of the next row
-            // the last pass already fetches the next image's first row (for the final image: a harmless
-            // re-read of its own), so HBM stays busy through the redistribution and the column pass
-            if (it + 1 < 4) issue(v, img, it + 1, lane_off);
+            // v is dead after the first radix-4 stage: its registers become the landing zone of the next row;
+            // the last pass already fetches the next image's first row
+            if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
             else issue(v, pre, 0, pre_off);
-            fwd_pass1_lds_finish(bb, twrow, gg);
-            group_forward_finish<8>(gg, exch, r, T[it]);
+            fwd_pass1_lds_finish(bb, twrow_y, gg);
+            group_forward_finish<LOGY>(gg, exch_y, ty, T[it]);
         }
         __syncthreads();
 #pragma unroll
-        for (int it = 0; it < 4; ++it)
+        for (int it = 0; it < ITY; ++it)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) lds[(row0 + 64 * it) * TPITCH + r + 16 * s] = T[it][s];
+            for (int mm = 0; mm < MMY; ++mm) lds[(row0 + GY * it) * TPITCH + ty + LY * mm] = T[it][mm];
         __syncthreads();
-        // pass 2: columns (along X); group g owns column q = g, lane r holds rows r + 16 i
-        cpx z[4];
-        {
-            cpx c[16], gg[16];
+        // pass 2: columns (along X); group gx owns column q = gx, lane tx holds rows tx + LX i
+        cpx c[16];
+        if (tid < G::COLT) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) c[i] = lds[(r + 16 * i) * TPITCH + g];
-            __syncthreads();
-            fwd_pass1_lds(c, twrow, gg);
-            wave_lds_fence();
-#pragma unroll
-            for (int q = 0; q < 16; ++q) exch[r * 17 + q] = gg[q];
-            wave_lds_fence();
-            cpx u[16];
-#pragma unroll
-            for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + r];
-            dft16_first4<-1>(u, z);
+            for (int i = 0; i < 16; ++i) c[i] = lds[(tx + LX * i) * TPITCH + gx];
         }
-        // lane order of the retained modes: element s*1024 + q*16 + r  <->  mode (p = r + 16 s, q)
-        // written through as it is produced, so the end-of-kernel cache write-back has nothing left to flush
-        float2* dst = spec + img * 4096;
+        __syncthreads();
+        if (tid < G::COLT) {
+            cpx gg[16], z[MMX];
+            fwd_pass1_lds(c, twrow_x, gg);
+            group_forward_finish<LOGX>(gg, exch_x, tx, z);
+            // lane order of the retained modes: element mm*COLT + q*LX + tx  <->  mode (p = tx + LX mm, q).
+            // Written through as it is produced, so the end-of-kernel cache write-back has nothing left to flush
+            float2* dst = spec + img * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) store_streaming(dst + tid + 1024 * s, z[s]);
+            for (int mm = 0; mm < MMX; ++mm) store_streaming(dst + tid + G::COLT * mm, z[mm]);
+        }
     }
 }
 
 // Backward image kernel, mirror of the forward one: persistent blocks, 16 waves per CU, twiddles in LDS.
-// The 32 KiB spectrum of the next image is fetched (4 registers per lane) while the current image's rows
+// The 32 KiB spectrum of the next image is fetched (a few registers per lane) while the current image's rows
 // are being transformed and stored, so a CU never waits for its input between images.
-__global__ __launch_bounds__(1024) void ifft2d_pad_256_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
-                                                              int nimg)
+template <int LOGX, int LOGY>
+__global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
+                                                          int nimg)
 {
+    using G = Geo2D<LOGX, LOGY>;
+    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, GY = G::GY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, j = lane >> 4, r = lane & 15, g = tid >> 4;
-    float2* exch = lds + g * EXCH256;
-    float2* twtab = lds + LDS2D_ELEMS;
-    fill_lds_twiddles<8>(twtab, tid, 1024);
-    const float2* twrow = twtab + r * kTwLdsPitch;
+    const int tid = threadIdx.x;
+    const int gy = tid / LY, ty = tid % LY;
+    const int gx = tid / LX, tx = tid % LX;
+    float2* exch_y = lds + gy * (LY * 17);
+    float2* exch_x = lds + gx * (LX * 17);
+    float2* twtab_y = lds + G::LDS_MAIN;
+    float2* twtab_x = twtab_y + kTwLdsSize;
+    fill_lds_twiddles<LOGY>(twtab_y, tid, 1024);
+    fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
+    const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
+    const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
     __syncthreads();
 
-    const int row0 = row_of(w, j, 0);
-    const unsigned lane_off = (unsigned)(row0 * IMG + r);
+    const int row0 = row_in_pass<LY>(gy);
+    const unsigned lane_off = (unsigned)(row0 * DY + ty);
+    const bool col_thread = tid < G::COLT;
 
     long img = blockIdx.x;
-    cpx c[4];
-    if (img < nimg) {
+    cpx c[MMX];
+    if (img < nimg && col_thread) {
         const float2* src = spec + img * 4096;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) c[s] = src[(unsigned)tid + 1024u * s];
+        for (int mm = 0; mm < MMX; ++mm) c[mm] = src[tid + G::COLT * mm];
     }
     for (; img < nimg; img += gridDim.x) {
         const long pre = img + gridDim.x < nimg ? img + gridDim.x : img;
-        // pass 1: columns (p -> x) of column q = g
-        {
-            cpx u[16];
-            group_backward256_lds(c, twrow, exch, r, u);
-            __syncthreads();
+        // pass 1: columns (p -> x) of column q = gx
+        cpx u[16];
+        if (col_thread) group_backward_lds<LOGX>(c, twrow_x, exch_x, tx, u);
+        // the exchange regions alias the tile: every wave must be done with them before the tile is written
+        __syncthreads();
+        if (col_thread) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) lds[(r + 16 * i) * TPITCH + g] = u[i];
-        }
-        // next image's spectrum (for the last image: a harmless re-read of its own)
-        {
+            for (int i = 0; i < 16; ++i) lds[(tx + LX * i) * TPITCH + gx] = u[i];
+            // next image's spectrum (for the last image: a harmless re-read of its own 32 KiB)
             const float2* src = spec + pre * 4096;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) c[s] = src[(unsigned)tid + 1024u * s];
+            for (int mm = 0; mm < MMX; ++mm) c[mm] = src[tid + G::COLT * mm];
         }
         __syncthreads();
-        cpx cc[4][4];
+        cpx cc[ITY][MMY];
 #pragma unroll
-        for (int it = 0; it < 4; ++it)
+        for (int it = 0; it < ITY; ++it)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) cc[it][s] = lds[(row0 + 64 * it) * TPITCH + r + 16 * s];
+            for (int mm = 0; mm < MMY; ++mm) cc[it][mm] = lds[(row0 + GY * it) * TPITCH + ty + LY * mm];
         __syncthreads();
-        // pass 2: rows (q -> y), coalesced 2 KiB row stores.
+        // pass 2: rows (q -> y), coalesced row stores.
         // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
         // dirty lines from lingering in the Infinity Cache and being written back under the next kernel's reads
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
+        for (int it = 0; it < ITY; ++it) {
             cpx yv[16];
-            group_backward256_lds(cc[it], twrow, exch, r, yv);
-            float2* dst = y + (img * IMG + 64 * it) * (long)IMG;   // uniform base + lane offset + immediates
+            group_backward_lds<LOGY>(cc[it], twrow_y, exch_y, ty, yv);
+            float2* dst = y + (img * DX + GY * it) * (long)DY;   // uniform base + lane offset + immediates
 #pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + 16 * i, yv[i]);
+            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + LY * i, yv[i]);
         }
     }
 }
@@ -300,35 +320,48 @@ static int cu_count()
     return cus;
 }
 
-hipError_t launch_fft2d_trunc_256(const float2* x, float2* spec, long nimg, hipStream_t stream)
+template <int LOGX, int LOGY>
+static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, long nimg, hipStream_t stream)
 {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fft2d_trunc_256_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_FWD_BYTES);
+    using G = Geo2D<LOGX, LOGY>;
+    static bool attr_set[2] = { false, false };
+    const void* fn = inverse ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY>)
+                             : reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>);
+    if (!attr_set[inverse]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
         if (e != hipSuccess) return e;
-        attr_set = true;
+        attr_set[inverse] = true;
     }
-    // one persistent block per CU (the LDS tile allows exactly one resident block per CU)
+    // persistent blocks: at most as many as fit at once (LDS allows one or two 1024-thread blocks per CU,
+    // the thread count exactly one)
     const long blocks = nimg < cu_count() ? nimg : cu_count();
-    hipLaunchKernelGGL(fft2d_trunc_256_kernel, dim3((unsigned)blocks), dim3(1024), LDS2D_FWD_BYTES, stream, x, spec,
-                       (int)nimg);
+    if (inverse)
+        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
+                           out, (int)nimg);
+    else
+        hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
+                           out, (int)nimg);
     return hipGetLastError();
 }
 
-hipError_t launch_ifft2d_pad_256(const float2* spec, float2* y, long nimg, hipStream_t stream)
+static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, const float2* in, float2* out, long nimg,
+                                        hipStream_t stream)
 {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ifft2d_pad_256_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS2D_FWD_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
-    const long blocks = nimg < cu_count() ? nimg : cu_count();
-    hipLaunchKernelGGL(ifft2d_pad_256_kernel, dim3((unsigned)blocks), dim3(1024), LDS2D_FWD_BYTES, stream, spec, y,
-                       (int)nimg);
-    return hipGetLastError();
+    if (logDX == 8 && logDY == 8) return launch_image_kernel<8, 8>(inverse, in, out, nimg, stream);
+    if (logDX == 8 && logDY == 7) return launch_image_kernel<8, 7>(inverse, in, out, nimg, stream);
+    if (logDX == 7 && logDY == 8) return launch_image_kernel<7, 8>(inverse, in, out, nimg, stream);
+    if (logDX == 7 && logDY == 7) return launch_image_kernel<7, 7>(inverse, in, out, nimg, stream);
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, long nimg, hipStream_t stream)
+{
+    return dispatch_image_kernel(false, logDX, logDY, x, spec, nimg, stream);
+}
+
+hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, long nimg, hipStream_t stream)
+{
+    return dispatch_image_kernel(true, logDX, logDY, spec, y, nimg, stream);
 }
 
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
