@@ -83,7 +83,7 @@ def main():
         torch.cuda.synchronize()
         for s in range(args.steps):
             ev[s][0].record(); tf.fft2d_trunc(x, spec)
-            ev[s][1].record(); tf.cgemm(bs * 4096, N, K, spec, W, cspec, 1.0)
+            ev[s][1].record(); tf.cgemm(bs * 4096, N, K, spec, W, cspec, 1.0, 0.0)
             ev[s][2].record(); tf.ifft2d_pad(cspec, y)
             ev[s][3].record()
         torch.cuda.synchronize()

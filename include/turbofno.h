@@ -94,16 +94,39 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
  * The 4096 retained modes of an image are stored in an order private to these two kernels (element
  * mm*(4*DX) + q*(DX/16) + t holds mode (p = t + (DX/16)*mm, q)); a GEMM over the channel dimension does
  * not care. Requires DX, DY in {128, 256}.
- *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] (column major, lda = M, ldb = K,
- *   ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
- *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:182-200) for beta = 0,
- *   the only value with which the fused variant D uses the product. Requires M % 256 == 0, M < 2^27,
+ *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] + beta * C[m + n*M] (column major,
+ *   lda = M, ldb = K, ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
+ *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:199), same argument order
+ *   (M, N, K, A, B, C, alpha, beta). C is read only when beta != 0. Requires M % 256 == 0, M < 2^27,
  *   N % 64 == 0, K % 8 == 0.
  */
 int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream);
 int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, void* stream);
 int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im,
-                   void* stream);
+                   float beta_re, float beta_im, void* stream);
+
+/*
+ * Stages of the unfused and half-fused variants (A, B, C), so that every executable of the reference's
+ * ablation can be rebuilt on this library.
+ *   turbofno_fft_stride_DY / turbofno_ifft_stride_DY replace the table entries fft_stride_DY[log2(DY)-7] and
+ *   ifft_stride_DY[log2(DY)-7], signature (float2* in, float2* out, int threadblock_bs, int total)
+ *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/fused.cu:27-28 tables, :195,:203 launches):
+ *     forward : in[total][DY] -> out[total][64]     backward: in[total][64] -> out[total][DY]
+ *   with `total` = number of contiguous signals (dimX * channels * bs).
+ *   turbofno_fused_fft_cgemm replaces fused_fft_cgemm[log2(DY)-7] of variant B
+ *   (fusion_variants/1D_B_exp_fused_fft_cgemm+ifft/fused_fft_cgemm_8.cuh:8, launch 1D_B.../fused.cu:141):
+ *     C[m + n*M] = alpha * sum_k FFT_trunc(x)[m + k*M] * W[k + n*K] + beta * C[m + n*M].
+ *   turbofno_fused_cgemm_ifft replaces fused_cgemm_ifft[log2(DY)-7] of variant C
+ *   (fusion_variants/1D_C_exp_fft+fused_cgemm_ifft/fused_cgemm_ifft_8.cuh:9, launch 1D_C.../fused.cu:144):
+ *     y = iFFT_pad(alpha * A * W), A[m + k*M] column major; C and beta are unused there and here.
+ * Same preconditions as turbofno_fused_fft_cgemm_ifft.
+ */
+int turbofno_fft_stride_DY(int logDY, const void* in, void* out, int threadblock_bs, long total, void* stream);
+int turbofno_ifft_stride_DY(int logDY, const void* in, void* out, int threadblock_bs, long total, void* stream);
+int turbofno_fused_fft_cgemm(int logDY, long M, int N, int K, const void* x, const void* W, void* C, float alpha_re,
+                             float alpha_im, float beta_re, float beta_im, void* stream);
+int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, const void* W, void* C, void* y,
+                              float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
 
 /* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
 const char* turbofno_last_error_string(void);

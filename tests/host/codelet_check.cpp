@@ -14,9 +14,12 @@ typedef std::complex<double> zd;
 
 static double frand() { return 2.0 * rand() / RAND_MAX - 1.0; }
 
-template <int LOGD> static double check_forward()
+template <int LOGD> static double check_forward(bool use_table)
 {
     constexpr int D = 1 << LOGD, L = D / 16;
+    alignas(16) static cpx table[kTwLdsSize];
+    for (int t = 0; t < L; ++t)
+        for (int r = 0; r < 16; ++r) table[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
     std::vector<cpx> x(D);
     for (auto& v : x) v = make_float2((float)frand(), (float)frand());
     // pass 1 per lane
@@ -25,7 +28,14 @@ template <int LOGD> static double check_forward()
         cpx v[16], tw[16], g[16];
         for (int i = 0; i < 16; ++i) v[i] = x[t + L * i];
         load_lane_twiddles<LOGD>(t, tw);
-        fwd_pass1(v, tw, g);
+        if (use_table) {
+            // the kernels' variant: twiddles from a pitch-18 table, transform split after the first radix-4 stage
+            cpx bb[16];
+            fft16_stage1<-1>(v, bb);
+            fwd_pass1_lds_finish(bb, table + t * kTwLdsPitch, g);
+        } else {
+            fwd_pass1(v, tw, g);
+        }
         for (int r = 0; r < 16; ++r) G[t * 16 + r] = g[r];
     }
     // pass 2 per output residue r
@@ -54,9 +64,12 @@ template <int LOGD> static double check_forward()
     return std::sqrt(num / den);
 }
 
-template <int LOGD> static double check_backward()
+template <int LOGD> static double check_backward(bool use_table)
 {
     constexpr int D = 1 << LOGD, L = D / 16;
+    alignas(16) static cpx table[kTwLdsSize];
+    for (int t = 0; t < L; ++t)
+        for (int r = 0; r < 16; ++r) table[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
     std::vector<cpx> C(64);
     for (auto& v : C) v = make_float2((float)frand(), (float)frand());
     std::vector<cpx> H(16 * L);  // H[r][t]
@@ -78,7 +91,8 @@ template <int LOGD> static double check_backward()
         cpx e[16], tw[16], out[16];
         for (int r = 0; r < 16; ++r) e[r] = H[r * L + t];
         load_lane_twiddles<LOGD>(t, tw);
-        inv_pass2(e, tw, out);
+        if (use_table) inv_pass2_lds(e, table + t * kTwLdsPitch, out);
+        else inv_pass2(e, tw, out);
         for (int i = 0; i < 16; ++i) y[t + L * i] = out[i];
     }
     double num = 0, den = 0;
@@ -95,8 +109,10 @@ template <int LOGD> static double check_backward()
 int main()
 {
     srand(12345);
-    double e[4] = { check_forward<8>(), check_forward<7>(), check_backward<8>(), check_backward<7>() };
-    printf("fwd256 %.3e fwd128 %.3e bwd256 %.3e bwd128 %.3e\n", e[0], e[1], e[2], e[3]);
+    double e[8] = { check_forward<8>(false), check_forward<7>(false), check_backward<8>(false), check_backward<7>(false),
+                    check_forward<8>(true),  check_forward<7>(true),  check_backward<8>(true),  check_backward<7>(true) };
+    printf("registers: fwd256 %.3e fwd128 %.3e bwd256 %.3e bwd128 %.3e\n", e[0], e[1], e[2], e[3]);
+    printf("table    : fwd256 %.3e fwd128 %.3e bwd256 %.3e bwd128 %.3e\n", e[4], e[5], e[6], e[7]);
     for (double v : e)
         if (!(v < 5e-7)) { printf("FAIL\n"); return 1; }
     printf("OK\n");

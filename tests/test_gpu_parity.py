@@ -105,3 +105,45 @@ def test_error_codes():
     with pytest.raises(tf.TurboFNOError) as e:
         tf.layer_1d(torch.zeros((8, 1, 2048), dtype=torch.complex64, device="cuda"), W)
     assert e.value.code == 2
+
+
+@pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128)])
+def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
+    """stages of variants A, B, C: contiguous transforms, cgemm with beta, the two half-fused kernels"""
+    print("case variant stages", S, DY, K, N, flush=True)
+    x, W = workloads.uniform_1d(S + DY + K, S, DY, K, N)
+    M = 64 * S
+    alpha, beta = 1 - 1j, -1 + 1j                       # the values the reference's drivers pass
+    # A = FFT_trunc(x): [K*S][DY] -> [K*S][64]  (= column-major M x K matrix)
+    A = torch.empty((K, S, 64), dtype=torch.complex64, device="cuda")
+    tf.fft_stride_DY(dev(x), A, 4, K * S)
+    torch.cuda.synchronize()
+    A_ref = oracle.fft_trunc_contig(x)
+    check(A, A_ref, tol, "fft_stride_DY")
+    # cgemm with beta: needs M % 256 == 0
+    A32 = A_ref.astype(np.complex64).reshape(K, M)
+    rng = np.random.default_rng(3)
+    C0 = (rng.uniform(-1, 1, (N, M)) + 1j * rng.uniform(-1, 1, (N, M))).astype(np.complex64)
+    if M % 256 == 0:
+        C = dev(C0.copy())
+        tf.cgemm(M, N, K, dev(A32), dev(W), C, alpha, beta)
+        torch.cuda.synchronize()
+        check(C, oracle.cgemm(A32, W, alpha) + beta * C0.astype(np.complex128), tol, "cgemm beta")
+    # variant B: fused FFT + CGEMM with beta
+    C = dev(C0.copy())
+    tf.fused_fft_cgemm(M, N, K, dev(x), dev(W), C, alpha, beta)
+    torch.cuda.synchronize()
+    C_ref = oracle.cgemm(A_ref.reshape(K, M), W, alpha) + beta * C0.astype(np.complex128)
+    check(C, C_ref, tol, "fused_fft_cgemm")
+    # backward stage of A and B: [N*S][64] -> [N*S][DY]
+    Cin = C_ref.astype(np.complex64).reshape(N, S, 64)
+    y = torch.empty((N, S, DY), dtype=torch.complex64, device="cuda")
+    tf.ifft_stride_DY(dev(Cin), y, 4, N * S)
+    torch.cuda.synchronize()
+    check(y, oracle.ifft_pad_contig(Cin.astype(np.complex128), DY), tol, "ifft_stride_DY")
+    # variant C: CGEMM + iFFT from the A matrix
+    y = torch.empty((N, S, DY), dtype=torch.complex64, device="cuda")
+    tf.fused_cgemm_ifft(M, N, K, dev(A32), dev(W), y, alpha)
+    torch.cuda.synchronize()
+    ref = oracle.ifft_pad_contig(oracle.cgemm(A32, W, alpha).reshape(N, S, 64), DY)
+    check(y, ref, tol, "fused_cgemm_ifft")

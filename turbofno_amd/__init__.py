@@ -12,8 +12,12 @@ from .api import (  # noqa: F401
     fft2d_trunc,
     ifft2d_pad,
     fft_stride,
+    fft_stride_DY,
+    fused_cgemm_ifft,
+    fused_fft_cgemm,
     fused_fft_cgemm_ifft,
     ifft_stride,
+    ifft_stride_DY,
     layer_1d,
     layer_2d,
     layer_2d_workspace_bytes,

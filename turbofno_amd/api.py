@@ -44,12 +44,17 @@ def lib():
         L.turbofno_layer_2d.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, vp, sz, i, vp]
         L.turbofno_fft2d_trunc.argtypes = [i, i, vp, vp, l, vp]
         L.turbofno_ifft2d_pad.argtypes = [i, i, vp, vp, l, vp]
-        L.turbofno_cgemm.argtypes = [l, i, i, vp, vp, vp, f, f, vp]
+        L.turbofno_cgemm.argtypes = [l, i, i, vp, vp, vp, f, f, f, f, vp]
+        L.turbofno_fft_stride_DY.argtypes = [i, vp, vp, i, l, vp]
+        L.turbofno_ifft_stride_DY.argtypes = [i, vp, vp, i, l, vp]
+        L.turbofno_fused_fft_cgemm.argtypes = [i, l, i, i, vp, vp, vp, f, f, f, f, vp]
+        L.turbofno_fused_cgemm_ifft.argtypes = [i, l, i, i, vp, vp, vp, vp, f, f, f, f, vp]
         L.turbofno_last_error_string.restype = ctypes.c_char_p
         L.turbofno_abi_version.restype = i
         for name in ("turbofno_fused_fft_cgemm_ifft", "turbofno_fft_stride", "turbofno_ifft_stride",
                      "turbofno_layer_1d", "turbofno_layer_2d", "turbofno_fft2d_trunc", "turbofno_ifft2d_pad",
-                     "turbofno_cgemm"):
+                     "turbofno_cgemm", "turbofno_fft_stride_DY", "turbofno_ifft_stride_DY", "turbofno_fused_fft_cgemm",
+                     "turbofno_fused_cgemm_ifft"):
             getattr(L, name).restype = i
         _LIB = L
     return _LIB
@@ -149,9 +154,39 @@ def ifft2d_pad(spec, y):
     return y
 
 
-def cgemm(M, N, K, A, B, C, alpha=1.0 + 0j):
-    """C[m + n*M] = alpha * sum_k A[m + k*M] B[k + n*K]  (A: [K][M], B: [N][K], C: [N][M] as tensors)."""
-    a = complex(alpha)
+def cgemm(M, N, K, A, B, C, alpha=1.0 + 0j, beta=0j):
+    """C[m + n*M] = alpha * sum_k A[m + k*M] B[k + n*K] + beta * C  (A: [K][M], B: [N][K], C: [N][M] as tensors)."""
+    a, b = complex(alpha), complex(beta)
     _check(lib().turbofno_cgemm(M, N, K, _dev_c64(A, "A"), _dev_c64(B, "B"), _dev_c64(C, "C"), a.real, a.imag,
-                                _stream()))
+                                b.real, b.imag, _stream()))
     return C
+
+
+def fft_stride_DY(inp, out, threadblock_bs, total):
+    """Contiguous truncated forward transform: in[total][DY] -> out[total][64]."""
+    _check(lib().turbofno_fft_stride_DY(_log2(inp.shape[-1]), _dev_c64(inp, "in"), _dev_c64(out, "out"),
+                                        threadblock_bs, total, _stream()))
+    return out
+
+
+def ifft_stride_DY(inp, out, threadblock_bs, total):
+    """Contiguous zero-padded backward transform: in[total][64] -> out[total][DY]."""
+    _check(lib().turbofno_ifft_stride_DY(_log2(out.shape[-1]), _dev_c64(inp, "in"), _dev_c64(out, "out"),
+                                         threadblock_bs, total, _stream()))
+    return out
+
+
+def fused_fft_cgemm(M, N, K, x, W, C, alpha=1.0 + 0j, beta=0j):
+    """Variant B's first kernel: C[N][M] = alpha * FFT_trunc(x) W + beta C, x: [K][S][DY]."""
+    a, b = complex(alpha), complex(beta)
+    _check(lib().turbofno_fused_fft_cgemm(_log2(x.shape[-1]), M, N, K, _dev_c64(x, "x"), _dev_c64(W, "W"),
+                                          _dev_c64(C, "C"), a.real, a.imag, b.real, b.imag, _stream()))
+    return C
+
+
+def fused_cgemm_ifft(M, N, K, A, W, y, alpha=1.0 + 0j):
+    """Variant C's second kernel: y[N][S][DY] = iFFT_pad(alpha * A W), A: [K][M]."""
+    a = complex(alpha)
+    _check(lib().turbofno_fused_cgemm_ifft(_log2(y.shape[-1]), M, N, K, _dev_c64(A, "A"), _dev_c64(W, "W"), None,
+                                           _dev_c64(y, "y"), a.real, a.imag, 0.0, 0.0, _stream()))
+    return y

@@ -125,14 +125,63 @@ int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, vo
     return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, (const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
 }
 
-int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im, void* stream)
+int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, float alpha_re, float alpha_im,
+                   float beta_re, float beta_im, void* stream)
 {
     if (!A || !B || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "A, B and C must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
     if (M % 256) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld is not a multiple of the 256-row block tile", M);
     if (M >= (1L << 27)) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld exceeds the 2^27 rows the 32-bit lane offsets cover", M);
     return hip_status(tfno::launch_cgemm_modes((const float2*)A, (const float2*)B, (float2*)C, M, N, K,
-                                               make_float2(alpha_re, alpha_im), (hipStream_t)stream), "cgemm launch");
+                                               make_float2(alpha_re, alpha_im), make_float2(beta_re, beta_im),
+                                               (hipStream_t)stream), "cgemm launch");
+}
+
+static int stride_DY_common(bool inverse, int logDY, const void* in, void* out, long total, void* stream)
+{
+    if (!in || !out) return fail(TURBOFNO_ERR_INVALID_ARG, "in and out must be non-null device pointers");
+    if (total <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "total=%ld must be positive", total);
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    hipError_t e = inverse ? tfno::launch_ifft_stride_DY(logDY, (const float2*)in, (float2*)out, total, (hipStream_t)stream)
+                           : tfno::launch_fft_stride_DY(logDY, (const float2*)in, (float2*)out, total, (hipStream_t)stream);
+    return hip_status(e, inverse ? "ifft_stride_DY launch" : "fft_stride_DY launch");
+}
+
+int turbofno_fft_stride_DY(int logDY, const void* in, void* out, int threadblock_bs, long total, void* stream)
+{
+    (void)threadblock_bs;
+    return stride_DY_common(false, logDY, in, out, total, stream);
+}
+
+int turbofno_ifft_stride_DY(int logDY, const void* in, void* out, int threadblock_bs, long total, void* stream)
+{
+    (void)threadblock_bs;
+    return stride_DY_common(true, logDY, in, out, total, stream);
+}
+
+int turbofno_fused_fft_cgemm(int logDY, long M, int N, int K, const void* x, const void* W, void* C, float alpha_re,
+                             float alpha_im, float beta_re, float beta_im, void* stream)
+{
+    if (!x || !W || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and C must be non-null device pointers");
+    if (int rc = check_gemm_dims(M, N, K)) return rc;
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
+    return hip_status(tfno::launch_fused_fft_cgemm(logDY, M / 64, N, K, (const float2*)x, (const float2*)W, (float2*)C,
+                                                   make_float2(alpha_re, alpha_im), make_float2(beta_re, beta_im),
+                                                   (hipStream_t)stream), "fused_fft_cgemm launch");
+}
+
+int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, const void* W, void* C, void* y,
+                              float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream)
+{
+    (void)C; (void)beta_re; (void)beta_im;
+    if (!A || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "A, W and y must be non-null device pointers");
+    if (int rc = check_gemm_dims(M, N, K)) return rc;
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
+    return hip_status(tfno::launch_fused_cgemm_ifft(logDY, M / 64, N, K, (const float2*)A, (const float2*)W, (float2*)y,
+                                                    make_float2(alpha_re, alpha_im), (hipStream_t)stream),
+                      "fused_cgemm_ifft launch");
 }
 
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo)
@@ -167,7 +216,7 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
         float2* spec = (float2*)ws;
         float2* cspec = (float2*)(ws + align256((size_t)K * bs * 4096 * sizeof(float2)));
         if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, (long)K * bs, st), "fft2d_trunc launch")) return rc;
-        if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, st), "cgemm_modes launch")) return rc;
+        if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, make_float2(0.f, 0.f), st), "cgemm_modes launch")) return rc;
         return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, (long)N * bs, st), "ifft2d_pad launch");
     }
     float2* t1 = (float2*)ws;

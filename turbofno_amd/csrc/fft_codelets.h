@@ -18,6 +18,7 @@
 // Plain-C++ build of the same arithmetic for the CPU unit test of the codelets (no HIP runtime).
 #include <cmath>
 struct float2 { float x, y; };
+struct alignas(16) float4 { float x, y, z, w; };
 static inline float2 make_float2(float x, float y) { return float2{ x, y }; }
 #define TFNO_DEV static inline
 #define TFNO_TABLE static const

@@ -227,7 +227,7 @@ constexpr int GEMM_MBLOCK = 256;    // m per block
 
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
                                                                    const float2* __restrict__ W, float2* __restrict__ C,
-                                                                   long Mtot, int N, int K, float2 alpha)
+                                                                   long Mtot, int N, int K, float2 alpha, float2 beta)
 {
     // sW[(k/4)*1024 + ((k&3)>>1)*512 + n'*4 + (k&1)*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:
     // {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1. In one operand read (16 n' x 4 channels) lanes 0-31 cover 256
@@ -303,8 +303,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        store_streaming(cblk + (long)(n0 + 8 * t) * Mtot + out_off, make_float2(acc[t][0], acc[t][1]));
-        store_streaming(cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off, make_float2(acc[t][2], acc[t][3]));
+        float2* p0 = cblk + (long)(n0 + 8 * t) * Mtot + out_off;
+        float2* p1 = cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off;
+        float2 r0 = make_float2(acc[t][0], acc[t][1]), r1 = make_float2(acc[t][2], acc[t][3]);
+        if (beta.x != 0.f || beta.y != 0.f) {          // C = alpha A W + beta C (the reference's cgemm / variant B)
+            r0 = cadd(r0, cmul(*p0, beta));
+            r1 = cadd(r1, cmul(*p1, beta));
+        }
+        store_streaming(p0, r0);
+        store_streaming(p1, r1);
     }
 }
 
@@ -365,11 +372,11 @@ hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y
 }
 
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
-                              hipStream_t stream)
+                              float2 beta, hipStream_t stream)
 {
     if (Mtot % GEMM_MBLOCK != 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)(Mtot / GEMM_MBLOCK), (unsigned)(N / 64), 1);
-    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha);
+    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha, beta);
     return hipGetLastError();
 }
 
