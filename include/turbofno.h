@@ -97,7 +97,7 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
  *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] + beta * C[m + n*M] (column major,
  *   lda = M, ldb = K, ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
  *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:199), same argument order
- *   (M, N, K, A, B, C, alpha, beta). C is read only when beta != 0. Requires M % 256 == 0, M < 2^27,
+ *   (M, N, K, A, B, C, alpha, beta). C is read only when beta != 0. Requires M % 64 == 0, M < 2^27,
  *   N % 64 == 0, K % 8 == 0.
  */
 int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, void* stream);

@@ -107,7 +107,7 @@ def test_error_codes():
     assert e.value.code == 2
 
 
-@pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128)])
+@pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128), (1, 128, 16, 64), (5, 256, 8, 64)])
 def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     """stages of variants A, B, C: contiguous transforms, cgemm with beta, the two half-fused kernels"""
     print("case variant stages", S, DY, K, N, flush=True)
@@ -120,15 +120,14 @@ def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     torch.cuda.synchronize()
     A_ref = oracle.fft_trunc_contig(x)
     check(A, A_ref, tol, "fft_stride_DY")
-    # cgemm with beta: needs M % 256 == 0
+    # cgemm with beta (M = 64*S: 64 and 320 exercise the partly filled last block of 256 rows)
     A32 = A_ref.astype(np.complex64).reshape(K, M)
     rng = np.random.default_rng(3)
     C0 = (rng.uniform(-1, 1, (N, M)) + 1j * rng.uniform(-1, 1, (N, M))).astype(np.complex64)
-    if M % 256 == 0:
-        C = dev(C0.copy())
-        tf.cgemm(M, N, K, dev(A32), dev(W), C, alpha, beta)
-        torch.cuda.synchronize()
-        check(C, oracle.cgemm(A32, W, alpha) + beta * C0.astype(np.complex128), tol, "cgemm beta")
+    C = dev(C0.copy())
+    tf.cgemm(M, N, K, dev(A32), dev(W), C, alpha, beta)
+    torch.cuda.synchronize()
+    check(C, oracle.cgemm(A32, W, alpha) + beta * C0.astype(np.complex128), tol, "cgemm beta")
     # variant B: fused FFT + CGEMM with beta
     C = dev(C0.copy())
     tf.fused_fft_cgemm(M, N, K, dev(x), dev(W), C, alpha, beta)

@@ -56,3 +56,36 @@ def test_driver_result_lines():
     lines = subprocess.run([exe2, cfg], check=True, capture_output=True, text=True, timeout=100).stdout.splitlines()
     got = [tuple(int(v) for v in re.findall(r"=(\d+)", ln)[:5]) for ln in lines]
     assert got == [(1, 128, 128, 64, 8), (1, 128, 128, 64, 16), (1, 256, 128, 64, 8), (1, 256, 128, 64, 16)], lines
+
+
+def _run_variant(exe, args):
+    env = dict(os.environ, TURBOFNO_DIGEST="1", TURBOFNO_NTEST="2")
+    r = subprocess.run([exe] + [str(a) for a in args], check=True, capture_output=True, text=True, timeout=100, env=env)
+    digest = [float(v) for v in re.search(r"digest: (\S+) (\S+) (\S+)", r.stderr).groups()]
+    return r.stdout, digest
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,args", [("1D", (4, 1, 128, 64, 16)), ("1D", (1, 1, 256, 128, 24)),
+                                      ("2D", (1, 128, 256, 64, 16)), ("2D", (2, 256, 128, 64, 8))])
+def test_all_variants_agree(dim, args):
+    # with TURBOFNO_DIGEST the ten executables reseed rand() per problem and see identical inputs: the staged (A), half-fused (B, C),
+    # fully fused (D) and library (E: hipFFT + hipBLAS) sequences must give the same output up to fp32 rounding.
+    # The first launch runs on a zeroed C, so beta does not enter.
+    bs, dx, dy, n, k = args
+    nelem = bs * dx * dy * n
+    xname = "DX" if dim == "2D" else "dimX"
+    ref = None
+    for v in "ABCDE":
+        exe = os.path.join(ROOT, "bin", f"TurboFNO_{dim}_{v}")
+        assert os.path.exists(exe), "build the drivers with make -C turbofno_amd/host"
+        print(exe, args, flush=True)
+        out, dg = _run_variant(exe, args)
+        assert re.fullmatch(rf"{dim}_{v}, bs={bs:<4d}, {xname}={dx:<4d}, DY={dy:<4d}, N={n:<4d}, K={k:<4d}, TIME=\s*\d+\.\d{{3}}ms\n", out), out
+        assert dg[2] > 0
+        if ref is None:
+            ref = dg
+            continue
+        scale = (ref[2] * nelem) ** 0.5          # bound of a weighted sum of nelem terms with that l2
+        assert abs(dg[2] - ref[2]) <= 1e-4 * ref[2], (v, dg, ref)
+        assert abs(dg[0] - ref[0]) <= 1e-5 * scale and abs(dg[1] - ref[1]) <= 1e-5 * scale, (v, dg, ref)

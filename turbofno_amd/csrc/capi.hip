@@ -130,7 +130,6 @@ int turbofno_cgemm(long M, int N, int K, const void* A, const void* B, void* C, 
 {
     if (!A || !B || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "A, B and C must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
-    if (M % 256) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld is not a multiple of the 256-row block tile", M);
     if (M >= (1L << 27)) return fail(TURBOFNO_ERR_INVALID_ARG, "M=%ld exceeds the 2^27 rows the 32-bit lane offsets cover", M);
     return hip_status(tfno::launch_cgemm_modes((const float2*)A, (const float2*)B, (float2*)C, M, N, K,
                                                make_float2(alpha_re, alpha_im), make_float2(beta_re, beta_im),

@@ -249,11 +249,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     // scalar base per k group + one 32-bit lane offset keeps the addresses out of the vector registers
     const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
     const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
+    const bool active = (long)blockIdx.x * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
     auto load_quarter = [&](float2 (&dst)[4], int kc, int kn, int quarter) {
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
             const int k4 = 16 * quarter + 4 * jj;            // lane reads channel kc + k4 + kq
-            dst[jj] = (k4 < kn) ? (blk + (long)(kc + k4) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+            dst[jj] = (active && k4 < kn) ? (blk + (long)(kc + k4) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         }
     };
 
@@ -282,6 +283,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
             *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
         }
         __syncthreads();
+        if (active) {
 #pragma unroll
         for (int quarter = 0; quarter < 4; ++quarter) {
             if (quarter + 1 < 4) load_quarter(bv[(quarter + 1) & 1], kc, kn, quarter + 1);
@@ -297,7 +299,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
                 }
             }
         }
+        }
     }
+    if (!active) return;
     // D[row = 4 kq + v][col]: row n' = 16 t + 4 kq + v = 2 n_local + c'  ->  n_local = 8 t + 2 kq + (v >> 1)
     float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
     const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
@@ -374,8 +378,8 @@ hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               float2 beta, hipStream_t stream)
 {
-    if (Mtot % GEMM_MBLOCK != 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
-    dim3 grid((unsigned)(Mtot / GEMM_MBLOCK), (unsigned)(N / 64), 1);
+    if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha, beta);
     return hipGetLastError();
 }

@@ -1,4 +1,8 @@
-// Drivers TurboFNO_1D_D and TurboFNO_2D_D: the fully fused 1D / 2D spectral layer, timed per problem.
+// Drivers TurboFNO_{1D,2D}_{A,B,C,D}: the spectral layer built from separately launched stages (A), with the
+// forward transform fused into the GEMM (B), with the backward transform fused into the GEMM (C), and fully
+// fused (D), each timed per problem. One source, selected by TURBOFNO_VARIANT / TURBOFNO_VARIANT_2D.
+// Stage sequences follow the reference's mains: 1D_A.../fused.cu:195-203, 1D_B.../fused.cu:141-144,
+// 1D_C.../fused.cu:139-144, 2D_A.../fused_trunc_2D.cu:189-219, 2D_B...:183-197, 2D_C...:184-199.
 //
 // Surface kept from the reference (fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:20-151,
 // fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:33-208):
@@ -7,7 +11,7 @@
 //   * alternatively five positional integers "<bs> <dimX|DX> <DY> <N> <K>" run a single problem
 //     (fusion_variants_benchmark/1D_D_exp_fused_fft_cgemm_ifft/fused.cu:33-46), or one argument
 //     names another config file (documented at README.md:122-132);
-//   * inputs: +-{0..9}e-3 from rand(); alpha = (1,-1);
+//   * inputs: +-{0..9}e-3 from rand(); alpha = (1,-1), beta = (-1,1) on a zeroed C (variants A and B use beta);
 //   * timing: one warm-up, then ntest x (launch + device synchronise) between two events, mean;
 //   * one result line per problem, format identical to fused.cu:146-147 / fused_trunc_2D.cu:203-204.
 // Differences: device buffers are sized per problem (the reference allocates once for its largest
@@ -15,11 +19,15 @@
 #include "../../include/turbofno.h"
 #include "TurboFNO.h"
 #include "utils.h"
+#include <cmath>
 #include <cstring>
 #include <string>
 
 #ifndef TURBOFNO_VARIANT_2D
 #define TURBOFNO_VARIANT_2D 0
+#endif
+#ifndef TURBOFNO_VARIANT
+#define TURBOFNO_VARIANT 'D'
 #endif
 #ifndef DEFAULT_CONFIG_PATH
 #define DEFAULT_CONFIG_PATH "benchmark_config/problem_size_1d.txt"
@@ -57,6 +65,7 @@ int main(int argc, char** argv)
         const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
         float* hx = (float*)malloc(sizeof(float) * 2 * in_elems);
         float* hw = (float*)malloc(sizeof(float) * 2 * w_elems);
+        if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
         generate_random_vector(hx, 2 * (long)in_elems);
         generate_random_vector(hw, 2 * (long)w_elems);
         void *dx = nullptr, *dw = nullptr, *dy = nullptr, *dws = nullptr;
@@ -66,21 +75,60 @@ int main(int argc, char** argv)
         HIP_RT_CALL(hipMemcpy(dx, hx, sizeof(float) * 2 * in_elems, hipMemcpyHostToDevice));
         HIP_RT_CALL(hipMemcpy(dw, hw, sizeof(float) * 2 * w_elems, hipMemcpyHostToDevice));
         size_t ws_bytes = 0;
-        if (TURBOFNO_VARIANT_2D) {
+        if (TURBOFNO_VARIANT_2D && TURBOFNO_VARIANT == 'D') {
             ws_bytes = turbofno_layer_2d_workspace_bytes(p.bs, p.dx, p.dy, p.k, p.n, algo);
             HIP_RT_CALL(hipMalloc(&dws, ws_bytes ? ws_bytes : 256));
         }
+        // stage buffers of the unfused / half-fused variants: A[M x K], C[M x N] and, in 2D, the X-stage
+        // intermediates t1[K*bs][64][DY], t2[N*bs][64][DY]
+        const long S = TURBOFNO_VARIANT_2D ? (long)p.bs * 64 : (long)p.bs * p.dx;   // signals per channel of the Y stage
+        const long M = 64 * S;
+        const int logDY = (int)lround(log2((double)p.dy)), logDX = (int)lround(log2((double)p.dx));
+        void *dA = nullptr, *dC = nullptr, *t1 = nullptr, *t2 = nullptr;
+        if (TURBOFNO_VARIANT != 'D') {
+            HIP_RT_CALL(hipMalloc(&dA, sizeof(float) * 2 * M * p.k));
+            HIP_RT_CALL(hipMalloc(&dC, sizeof(float) * 2 * M * p.n));
+            HIP_RT_CALL(hipMemset(dC, 0, sizeof(float) * 2 * M * p.n));
+            if (TURBOFNO_VARIANT_2D) {
+                HIP_RT_CALL(hipMalloc(&t1, sizeof(float) * 2 * S * p.dy * p.k));
+                HIP_RT_CALL(hipMalloc(&t2, sizeof(float) * 2 * S * p.dy * p.n));
+            }
+        }
+        const float beta_re = -1.0f, beta_im = 1.0f;
         auto launch = [&]() {
+            const void* yin = dx;            // input of the Y stage
+            void* yout = dy;                 // output of the Y stage
+            if (TURBOFNO_VARIANT == 'D') {
+                if (TURBOFNO_VARIANT_2D)
+                    CHECK_TURBOFNO(turbofno_layer_2d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, dws, ws_bytes, algo, nullptr));
+                else
+                    CHECK_TURBOFNO(turbofno_layer_1d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, nullptr));
+                return;
+            }
+            if (TURBOFNO_VARIANT_2D) {
+                CHECK_TURBOFNO(turbofno_fft_stride(logDX, dx, t1, threadblock_bs, p.dy, (long)p.dy * p.k * p.bs, 64, nullptr));
+                yin = t1; yout = t2;
+            }
+            if (TURBOFNO_VARIANT == 'A') {
+                CHECK_TURBOFNO(turbofno_fft_stride_DY(logDY, yin, dA, threadblock_bs, S * p.k, nullptr));
+                CHECK_TURBOFNO(turbofno_cgemm(M, p.n, p.k, dA, dw, dC, alpha_re, alpha_im, beta_re, beta_im, nullptr));
+                CHECK_TURBOFNO(turbofno_ifft_stride_DY(logDY, dC, yout, threadblock_bs, S * p.n, nullptr));
+            } else if (TURBOFNO_VARIANT == 'B') {
+                CHECK_TURBOFNO(turbofno_fused_fft_cgemm(logDY, M, p.n, p.k, yin, dw, dC, alpha_re, alpha_im, beta_re, beta_im, nullptr));
+                CHECK_TURBOFNO(turbofno_ifft_stride_DY(logDY, dC, yout, threadblock_bs, S * p.n, nullptr));
+            } else {
+                CHECK_TURBOFNO(turbofno_fft_stride_DY(logDY, yin, dA, threadblock_bs, S * p.k, nullptr));
+                CHECK_TURBOFNO(turbofno_fused_cgemm_ifft(logDY, M, p.n, p.k, dA, dw, dC, yout, alpha_re, alpha_im, beta_re, beta_im, nullptr));
+            }
             if (TURBOFNO_VARIANT_2D)
-                CHECK_TURBOFNO(turbofno_layer_2d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, dws, ws_bytes, algo, nullptr));
-            else
-                CHECK_TURBOFNO(turbofno_layer_1d(p.bs, p.dx, p.dy, p.k, p.n, dx, dw, dy, alpha_re, alpha_im, nullptr));
+                CHECK_TURBOFNO(turbofno_ifft_stride(logDX, t2, dy, threadblock_bs, p.dy, (long)p.dy * p.n * p.bs, 64, nullptr));
         };
         HIP_RT_CALL(hipDeviceSynchronize());
         launch();
         CHECK_HIP_KERNEL();
         HIP_RT_CALL(hipDeviceSynchronize());
         CHECK_HIP_KERNEL();
+        if (getenv("TURBOFNO_DIGEST")) print_output_digest(dy, out_elems);
 
         hipEvent_t t_begin, t_end;
         float elapsed_time = 0.f;
@@ -96,14 +144,18 @@ int main(int argc, char** argv)
         HIP_RT_CALL(hipEventElapsedTime(&elapsed_time, t_begin, t_end));
         elapsed_time /= ntest;
         if (TURBOFNO_VARIANT_2D)
-            printf("2D_D, bs=%-4d, DX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
+            printf("2D_%c, bs=%-4d, DX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", TURBOFNO_VARIANT, p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
         else
-            printf("1D_D, bs=%-4d, dimX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
+            printf("1D_%c, bs=%-4d, dimX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", TURBOFNO_VARIANT, p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
         fflush(stdout);
         HIP_RT_CALL(hipEventDestroy(t_begin));
         HIP_RT_CALL(hipEventDestroy(t_end));
         HIP_RT_CALL(hipFree(dx)); HIP_RT_CALL(hipFree(dw)); HIP_RT_CALL(hipFree(dy));
         if (dws) HIP_RT_CALL(hipFree(dws));
+        if (dA) HIP_RT_CALL(hipFree(dA));
+        if (dC) HIP_RT_CALL(hipFree(dC));
+        if (t1) HIP_RT_CALL(hipFree(t1));
+        if (t2) HIP_RT_CALL(hipFree(t2));
         free(hx); free(hw);
     }
     return 0;

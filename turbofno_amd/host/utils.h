@@ -19,6 +19,12 @@ std::map<std::string, std::vector<int>> load_problem_config(const std::string& p
 // +-{0..9} * 1e-3 from rand(), unseeded: the reference's input distribution
 void generate_random_vector(float* target, long n);
 
+// With TURBOFNO_DIGEST set in the environment the drivers print, after the warm-up launch of each problem, one
+// line "digest: <weighted sum re> <weighted sum im> <sum |y|^2>" of the output on stderr, and reseed rand() before
+// generating each problem's inputs: every variant of a problem then sees the same inputs and must print the same
+// digest up to fp32 rounding.
+void print_output_digest(const void* device_y, size_t complex_elems);
+
 #define HIP_RT_CALL(call)                                                                                    \
     do {                                                                                                     \
         hipError_t status_ = (call);                                                                         \
