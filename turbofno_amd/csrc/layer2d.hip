@@ -213,10 +213,11 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 // expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition) on
 // v_mfma_f32_16x16x4_f32: rows = (n, re/im), cols = 16 consecutive m, contraction = 4 channels x re|im.
 // A block is 16 waves; wave w owns the 16-m strip w and the whole 64-channel n tile (8 accumulators of
-// 16x16), so every element of A is loaded exactly once. One float2 load per lane feeds two matrix
-// instructions per n tile (real parts, then imaginary parts). The K loop runs in quarters whose loads are
-// issued one quarter ahead; the four waves of a SIMD get descending priorities so that they finish
-// staggered and the stores of one drain under the matrix work of the others.
+// 16x16), so every element of A is loaded exactly once: the strip of a 64-channel chunk sits in 16 float2
+// registers per lane, all loads in flight while the W tile is built. One float2 of A feeds two matrix
+// instructions per n tile (real parts, then imaginary parts). The n tiles are the outer loop, so each is
+// stored as soon as it is complete and its stores drain under the matrix work of the next ones; the four
+// waves of a SIMD get descending priorities so that they run staggered.
 // ---------------------------------------------------------------------------------------------
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -250,18 +251,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
     const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
     const bool active = (long)blockIdx.x * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
-    auto load_quarter = [&](float2 (&dst)[4], int kc, int kn, int quarter) {
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const int k4 = 16 * quarter + 4 * jj;            // lane reads channel kc + k4 + kq
-            dst[jj] = (active && k4 < kn) ? (blk + (long)(kc + k4) * Mtot)[lane_off] : make_float2(0.f, 0.f);
-        }
-    };
+    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
+    const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
+    const bool has_beta = beta.x != 0.f || beta.y != 0.f;
 
     for (int kc = 0; kc < K; kc += GEMM_KC) {
         const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;   // multiple of 8 (caller contract)
-        float2 bv[2][4];
-        load_quarter(bv[0], kc, kn, 0);
+        const bool last = kc + GEMM_KC >= K;
+        // the wave's whole A strip of this chunk: lane (kq, col) holds channels kc + 4 g + kq, g = 0..15
+        float2 bv[GEMM_KC / 4];
+#pragma unroll
+        for (int g = 0; g < GEMM_KC / 4; ++g)
+            bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         __syncthreads();
         // W tile: lanes run along k, the contiguous direction of W[k + n*K], so a wave reads 512 contiguous bytes
         // (the LDS stores then collide on banks, but there are only eight of them per lane)
@@ -283,39 +284,31 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
             *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
         }
         __syncthreads();
-        if (active) {
+        if (!active) continue;
+        // n tile outermost: a tile is complete after its 2 * kn / 4 matrix instructions and, in the last chunk, is
+        // stored at once, so its stores drain under the matrix work of the following tiles
 #pragma unroll
-        for (int quarter = 0; quarter < 4; ++quarter) {
-            if (quarter + 1 < 4) load_quarter(bv[(quarter + 1) & 1], kc, kn, quarter + 1);
+        for (int t = 0; t < 8; ++t) {
+            const float* wrow = &sW[(kq >> 1) * 512 + (t * 16 + col) * 4 + (kq & 1) * 2];
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const int kg = 4 * quarter + jj;             // channel group; this lane's channel is 4 kg + kq
-                const float2 b = bv[quarter & 1][jj];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float2 a = *reinterpret_cast<const float2*>(&sW[kg * GEMM_WGROUP + (kq >> 1) * 512 + (t * 16 + col) * 4 + (kq & 1) * 2]);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[t], 0, 0, 0);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[t], 0, 0, 0);
+            for (int g = 0; g < GEMM_KC / 4; ++g) {
+                const float2 a = *reinterpret_cast<const float2*>(wrow + g * GEMM_WGROUP);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, bv[g].x, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, bv[g].y, acc[t], 0, 0, 0);
+            }
+            if (last) {
+                // D[row = 4 kq + v][col]: row n' = 16 t + 4 kq + v = 2 n_local + c'  ->  n_local = 8 t + 2 kq + (v >> 1)
+                float2* p0 = cblk + (long)(n0 + 8 * t) * Mtot + out_off;
+                float2* p1 = cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off;
+                float2 r0 = make_float2(acc[t][0], acc[t][1]), r1 = make_float2(acc[t][2], acc[t][3]);
+                if (has_beta) {          // C = alpha A W + beta C (the reference's cgemm / variant B)
+                    r0 = cadd(r0, cmul(*p0, beta));
+                    r1 = cadd(r1, cmul(*p1, beta));
                 }
+                *p0 = r0;                // plain stores: the backward kernel reads C back through the caches
+                *p1 = r1;
             }
         }
-        }
-    }
-    if (!active) return;
-    // D[row = 4 kq + v][col]: row n' = 16 t + 4 kq + v = 2 n_local + c'  ->  n_local = 8 t + 2 kq + (v >> 1)
-    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
-    const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        float2* p0 = cblk + (long)(n0 + 8 * t) * Mtot + out_off;
-        float2* p1 = cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off;
-        float2 r0 = make_float2(acc[t][0], acc[t][1]), r1 = make_float2(acc[t][2], acc[t][3]);
-        if (beta.x != 0.f || beta.y != 0.f) {          // C = alpha A W + beta C (the reference's cgemm / variant B)
-            r0 = cadd(r0, cmul(*p0, beta));
-            r1 = cadd(r1, cmul(*p1, beta));
-        }
-        store_streaming(p0, r0);
-        store_streaming(p1, r1);
     }
 }
 
