@@ -43,6 +43,25 @@ def test_layer_1d(bs, DY, K, N, alpha, tol):
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d")
 
 
+@pytest.mark.parametrize("algo", [1, 2])
+@pytest.mark.parametrize("bs,DY,K,N,alpha", [
+    (2, 256, 32, 64, 1.0),           # exactly one chunk of the matrix-core kernel
+    (3, 256, 72, 128, 1 - 1j),       # chunks 32 + 32 + 8, two N tiles
+    (2, 256, 8, 64, 1.0),            # K smaller than a chunk
+    (4, 128, 64, 64, 1.0),           # DY=128: one chunk of 64 channels
+    (3, 128, 72, 128, 0.5j),         # DY=128: 64 + 8
+    (2, 256, 128, 128, 1.0),         # large-hidden shape
+])
+def test_layer_1d_both_contractions(bs, DY, K, N, alpha, algo, tol, monkeypatch):
+    """the SIMT and the matrix-core fused kernels, forced through TURBOFNO_1D_ALGO, on the same problems"""
+    print("case layer_1d algo", algo, bs, DY, K, N, alpha, flush=True)
+    monkeypatch.setenv("TURBOFNO_1D_ALGO", str(algo))
+    x, W = workloads.smooth_1d(11 + bs + DY + K, bs, DY, K, N)
+    y = tf.layer_1d(dev(x), dev(W), alpha=alpha)
+    torch.cuda.synchronize()
+    check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d algo %d" % algo)
+
+
 @pytest.mark.parametrize("DX,DY,nsig", [(128, 128, 3), (256, 128, 2), (128, 256, 2), (256, 256, 2)])
 def test_stride_stages(DX, DY, nsig, tol):
     print("case stride", DX, DY, nsig, flush=True)

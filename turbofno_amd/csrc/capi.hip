@@ -4,6 +4,7 @@
 #include "kernels.h"
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 
 namespace {
 
@@ -59,6 +60,15 @@ int turbofno_abi_version(void) { return 1; }
 
 const char* turbofno_last_error_string(void) { return g_err; }
 
+// The fused 1D entry point keeps the reference's kernel signature, which has no room for an algorithm selector:
+// TURBOFNO_1D_ALGO in the environment (0 by size, 1 SIMT contraction, 2 matrix cores) overrides the choice.
+static int algo_1d()
+{
+    const char* e = getenv("TURBOFNO_1D_ALGO");
+    const int a = e ? atoi(e) : 0;
+    return (a == 1 || a == 2) ? a : 0;
+}
+
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream)
 {
@@ -68,7 +78,7 @@ int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x
     if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
     if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
     hipError_t e = tfno::launch_fused_fft_cgemm_ifft(logDY, M / 64, N, K, (const float2*)x, (const float2*)W, (float2*)y,
-                                                     make_float2(alpha_re, alpha_im), (hipStream_t)stream);
+                                                     make_float2(alpha_re, alpha_im), algo_1d(), (hipStream_t)stream);
     return hip_status(e, "fused_fft_cgemm_ifft launch");
 }
 
@@ -221,7 +231,7 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     float2* t1 = (float2*)ws;
     float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));
     if (int rc = hip_status(tfno::launch_fft_stride(logDX, (const float2*)x, t1, DY, (long)K * bs, st), "fft_stride launch")) return rc;
-    if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, st), "fused_fft_cgemm_ifft launch")) return rc;
+    if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, algo_1d(), st), "fused_fft_cgemm_ifft launch")) return rc;
     return hip_status(tfno::launch_ifft_stride(logDX, t2, (float2*)y, DY, (long)N * bs, st), "ifft_stride launch");
 }
 

@@ -4,9 +4,13 @@
 
 namespace tfno {
 
+// compute units of the current device (cached)
+int cu_count();
+
 // 1D fused layer / Y stage of the three-kernel 2D pipeline. S = number of signals per channel.
+// algo: 0 = chosen by size, 1 = SIMT contraction, 2 = contraction on the matrix cores.
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
-                                       float2 alpha, hipStream_t stream);
+                                       float2 alpha, int algo, hipStream_t stream);
 
 // Halves of the fused kernel (variants B and C) and the stand-alone contiguous transforms (variant A).
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

@@ -122,6 +122,136 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
     }
 }
 
+// Fused 1D layer with the contraction on the fp32 matrix cores, for channel counts where the GEMM dominates the
+// arithmetic (K >= one chunk). Same operands, grid (S, N/64) and block-traverses-K schedule as the kernel above;
+// 512 threads = 8 waves:
+//   * a chunk is KC = 512/L channels (32 for DY=256, 64 for DY=128): every L-lane group transforms one channel and
+//     leaves its 64 modes in sA[k][m]; the loads of the next chunk are issued as soon as the first pass has consumed
+//     the registers, so they travel under the exchange, the W tile build and the matrix work;
+//   * C'[n'][m] += W'[n'][k'] A'[k'][m] is the 4-real form of the complex product on v_mfma_f32_16x16x4_f32:
+//     n' = (n, re|im) 128 rows, m 64 columns = 8 x 4 tiles, four per wave (one m tile, four n' tiles), so one read of
+//     A from LDS feeds eight matrix instructions. W' (alpha folded in) uses the conflict-free LDS order of
+//     cgemm_modes_kernel; sA has a pitch of 80 complex so that the two k rows a half wave reads fall on disjoint banks;
+//   * the product goes through LDS once (sC, pitch 72) to reach the lane groups that run the zero-padded backward
+//     transforms and store y.
+// sA aliases the exchange regions of the lane groups (the transforms of a chunk are complete before sA is written),
+// sC aliases the W' tile.
+typedef float floatx4_1d __attribute__((ext_vector_type(4)));
+
+template <int LOGDY> struct GeoMfma1D {
+    static constexpr int L = Geo1D<LOGDY>::L, MM = 64 / L;
+    static constexpr int THREADS = 512;
+    static constexpr int KC = THREADS / L;                    // channels per chunk = lane groups per block
+    static constexpr int PA = 80, PC = 72;                    // pitches (complex) of sA and sC
+    static constexpr int EXCH = L * 17;
+    static constexpr int REGION0 = KC * EXCH > KC * PA ? KC * EXCH : KC * PA;              // exchange | sA
+    static constexpr int REGION1 = KC * 128 > 64 * PC ? KC * 128 : 64 * PC;                // W' | sC   (complex)
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
+};
+
+template <int LOGDY>
+__global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
+                                                                  const float2* __restrict__ W, float2* __restrict__ y,
+                                                                  float2 alpha)
+{
+    using G = GeoMfma1D<LOGDY>;
+    constexpr int DY = 1 << LOGDY, L = G::L, MM = G::MM, KC = G::KC, PA = G::PA, PC = G::PC;
+    extern __shared__ float2 lds[];
+    float2* sA = lds;                                          // [KC][PA]; aliases the exchange regions
+    float* sW = reinterpret_cast<float*>(lds + G::REGION0);    // [(k/4)][(k&3)>>1][n' 128][k&1][c]
+    float2* sC = lds + G::REGION0;                             // [64][PC]; aliases sW after the K loop
+
+    const int tid = threadIdx.x;
+    const int g = tid / L, t = tid % L;                        // transform role: lane group = channel of the chunk
+    const int wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;   // matrix role
+    const int mt = wave & 3, nt0 = (wave >> 2) * 4;            // m tile, first of four n' tiles
+    const long s = blockIdx.x;
+    const int n0 = blockIdx.y * 64;
+    float2* exch = lds + g * G::EXCH;
+
+    cpx tw[16];
+    load_lane_twiddles<LOGDY>(t, tw);
+
+    floatx4_1d acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
+
+    auto issue = [&](cpx (&dst)[16], int k) {
+        const float2* src = x + ((long)k * S + s) * DY + t;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[i] = src[L * i];
+    };
+    cpx v[16];
+    if (g < K) issue(v, g);
+
+    for (int kc = 0; kc < K; kc += KC) {
+        const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
+        // W chunk: lanes run along k, the contiguous direction of W[k + n*K]
+        constexpr int WPT = KC * 64 / G::THREADS;
+        float2 wv[WPT];
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * G::THREADS;
+            const int k = idx % KC, n = idx / KC;
+            wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        }
+        cpx out[MM];
+        if (g < kn) {
+            cpx gg[16];
+            fwd_pass1(v, tw, gg);
+            if (kc + KC + g < K) issue(v, kc + KC + g);        // next chunk's channel of this group
+            group_forward_finish<LOGDY>(gg, exch, t, out);
+        }
+        __syncthreads();                                       // all exchanges done: sA may overwrite them
+        if (g < kn) {
+#pragma unroll
+            for (int a = 0; a < MM; ++a) sA[g * PA + t + L * a] = out[a];
+        }
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * G::THREADS;
+            const int k = idx % KC, n = idx / KC;
+            const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
+            float* dstw = &sW[(k >> 2) * 1024 + ((k & 3) >> 1) * 512 + (2 * n) * 4 + (k & 1) * 2];
+            *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
+            *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
+        }
+        __syncthreads();
+        const float2* arow = sA + kq * PA + mt * 16 + col;
+        const float* wrow = sW + (kq >> 1) * 512 + (nt0 * 16 + col) * 4 + (kq & 1) * 2;
+        for (int kg = 0; kg < kn / 4; ++kg) {
+            const float2 b = arow[kg * 4 * PA];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float2 a = *reinterpret_cast<const float2*>(wrow + kg * 1024 + i * 64);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[i], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                       // sA / sW are free again (next chunk, or sC below)
+    }
+
+    // D[row = 4 kq + v][col] of tile i: n' = 16 (nt0 + i) + 4 kq + v = 2 n + c'  ->  n = 8 (nt0 + i) + 2 kq + (v >> 1)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int n = 8 * (nt0 + i) + 2 * kq;
+        sC[n * PC + mt * 16 + col] = make_float2(acc[i][0], acc[i][1]);
+        sC[(n + 1) * PC + mt * 16 + col] = make_float2(acc[i][2], acc[i][3]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 64 / KC; ++pass) {
+        const int n = g + KC * pass;
+        cpx c[MM], yv[16];
+#pragma unroll
+        for (int a = 0; a < MM; ++a) c[a] = sC[n * PC + t + L * a];
+        group_backward<LOGDY>(c, tw, exch, t, yv);
+        float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+    }
+}
+
 // Stand-alone truncated forward / zero-padded backward transforms of contiguous signals (variants A, B, C):
 //   fft_stride_DY : in[nsig][DY] -> out[nsig][64]      ifft_stride_DY : in[nsig][64] -> out[nsig][DY]
 // Replace fft_N_stride_DY / ifft_N_stride_DY of the missing TurboFFT submodule (launched at
@@ -181,9 +311,34 @@ static hipError_t dispatch_fused_1d(int logDY, long S, int N, int K, const float
     }
 }
 
-hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
-                                       float2 alpha, hipStream_t stream)
+template <int LOGDY>
+static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                    hipStream_t stream)
 {
+    using G = GeoMfma1D<LOGDY>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY>), dim3((unsigned)S, (unsigned)(N / 64)), dim3(G::THREADS),
+                       G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
+    return hipGetLastError();
+}
+
+// algo: 0 = by size (matrix cores once K fills a chunk of the 512-thread kernel), 1 = SIMT kernel, 2 = matrix cores
+hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
+                                       float2 alpha, int algo, hipStream_t stream)
+{
+    // by size: the matrix-core kernel needs K to fill a chunk, and it keeps one 8-wave block per CU, so it wins while
+    // every block has a CU to itself (measured crossover: about one block per CU); beyond that the SIMT kernel's
+    // three blocks per CU hide more latency
+    const bool fills = (logDY == 8 && K >= 32) || (logDY == 7 && K >= 64);
+    const bool mfma = algo == 2 || (algo == 0 && fills && S * (N / 64) <= cu_count());
+    if (mfma && logDY == 8) return launch_fused_mfma<8>(S, N, K, x, W, y, alpha, stream);
+    if (mfma && logDY == 7) return launch_fused_mfma<7>(S, N, K, x, W, y, alpha, stream);
     return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream);
 }
 

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     }
 }
 
-static int cu_count()
+int cu_count()
 {
     static int cus = 0;
     if (!cus) {
