@@ -39,7 +39,7 @@ extern "C" {
 /* algorithms of turbofno_layer_2d */
 #define TURBOFNO_2D_AUTO          0
 #define TURBOFNO_2D_THREE_KERNEL  1  /* X transform, fused Y stage, X inverse: the reference's structure */
-#define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM (default)                */
+#define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM                          */
 
 /*
  * Fused 1D layer kernel. Replaces the table entries fused_fft_cgemm_ifft[log2(DY)-7]
@@ -48,7 +48,7 @@ extern "C" {
  *   (int M, int N, int K, float2* FFT_input, float2* B, float2* C, float2* FFT_output, float2 alpha, float2 beta))
  * M = 64 * S where S = bs*dimX signals per channel. `C` is unused by the reference kernel (its beta*C
  * term is commented out, fused_fft_cgemm_ifft_7.cuh:186-187) and may be NULL; beta is ignored.
- * Requires logDY in {7, 8}, M % 64 == 0, N % 64 == 0, K % 8 == 0 (utils/TurboFNO.h:2-4).
+ * Requires logDY in {7, 8, 9, 10}, M % 64 == 0, N % 64 == 0, K % 8 == 0 (utils/TurboFNO.h:2-4).
  */
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
@@ -60,7 +60,7 @@ int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x
  * forward : in[total/DY][DX][DY] -> out[total/DY][dimX][DY]   FFT along DX, first dimX rows kept
  * backward: in[total/DY][dimX][DY] -> out[total/DY][DX][DY]   rows >= dimX taken as zero, backward FFT along DX
  * `total` = number of columns (DY * channels * bs). threadblock_bs (columns per block in the
- * reference) is accepted for signature compatibility and ignored. Requires logDX in {7, 8},
+ * reference) is accepted for signature compatibility and ignored. Requires logDX in {7, 8, 9, 10},
  * dimX == 64, DY % 16 == 0, total % DY == 0.
  */
 int turbofno_fft_stride(int logDX, const void* in, void* out, int threadblock_bs, int DY, long total, int dimX,
@@ -80,7 +80,8 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:133-172). The reference keeps its
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
- * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE.
+ * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE once K*bs images fill the CUs, THREE_KERNEL below; the workspace query
+ * with the same arguments makes the same choice.
  */
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo);
 int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,

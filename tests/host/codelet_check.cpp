@@ -106,6 +106,49 @@ template <int LOGD> static double check_backward(bool use_table)
     return std::sqrt(num / den);
 }
 
+// lengths 512 / 1024: lanes emulated in a loop around the same exchange array the kernels use
+template <int LOGD> static double check_wide(bool backward)
+{
+    constexpr int D = 1 << LOGD, L = D / 16;
+    std::vector<cpx> exch(L * 17);
+    double num = 0, den = 0;
+    if (!backward) {
+        std::vector<cpx> x(D);
+        for (auto& v : x) v = make_float2((float)frand(), (float)frand());
+        for (int t = 0; t < L; ++t) {
+            cpx v[16], tw[16], g[16];
+            for (int i = 0; i < 16; ++i) v[i] = x[t + L * i];
+            load_lane_twiddles<LOGD>(t, tw);
+            fwd_pass1(v, tw, g);
+            for (int r = 0; r < 16; ++r) exch[t * 17 + r] = g[r];
+        }
+        for (int m = 0; m < 64; ++m) {
+            const cpx X = wide_forward_mode<L>(exch.data(), m);
+            zd acc = 0;
+            for (int j = 0; j < D; ++j) acc += zd(x[j].x, x[j].y) * std::polar(1.0, -2.0 * M_PI * ((long)j * m % D) / D);
+            num += std::norm(acc - zd(X.x, X.y));
+            den += std::norm(acc);
+        }
+    } else {
+        for (int m = 0; m < 64; ++m) exch[m] = make_float2((float)frand(), (float)frand());
+        std::vector<cpx> y(D);
+        for (int t = 0; t < L; ++t) {
+            cpx e[16], tw[16], out[16];
+            wide_backward_inputs<L>(exch.data(), t, e);
+            load_lane_twiddles<LOGD>(t, tw);
+            inv_pass2(e, tw, out);
+            for (int i = 0; i < 16; ++i) y[t + L * i] = out[i];
+        }
+        for (int j = 0; j < D; ++j) {
+            zd acc = 0;
+            for (int m = 0; m < 64; ++m) acc += zd(exch[m].x, exch[m].y) * std::polar(1.0, 2.0 * M_PI * ((long)j * m % D) / D);
+            num += std::norm(acc - zd(y[j].x, y[j].y));
+            den += std::norm(acc);
+        }
+    }
+    return std::sqrt(num / den);
+}
+
 int main()
 {
     srand(12345);
@@ -113,7 +156,11 @@ int main()
                     check_forward<8>(true),  check_forward<7>(true),  check_backward<8>(true),  check_backward<7>(true) };
     printf("registers: fwd256 %.3e fwd128 %.3e bwd256 %.3e bwd128 %.3e\n", e[0], e[1], e[2], e[3]);
     printf("table    : fwd256 %.3e fwd128 %.3e bwd256 %.3e bwd128 %.3e\n", e[4], e[5], e[6], e[7]);
+    double w[4] = { check_wide<9>(false), check_wide<10>(false), check_wide<9>(true), check_wide<10>(true) };
+    printf("wide     : fwd512 %.3e fwd1024 %.3e bwd512 %.3e bwd1024 %.3e\n", w[0], w[1], w[2], w[3]);
     for (double v : e)
+        if (!(v < 5e-7)) { printf("FAIL\n"); return 1; }
+    for (double v : w)
         if (!(v < 5e-7)) { printf("FAIL\n"); return 1; }
     printf("OK\n");
     return 0;

@@ -34,6 +34,9 @@ def check(got, ref, tol, what=""):
     (5, 256, 24, 64, 1.0),           # K not a multiple of the 16-channel chunk
     (16, 256, 32, 128, 0.5j),
     (64, 128, 16, 64, 1.0),
+    (3, 512, 24, 64, 1 - 1j),        # lengths 512 / 1024: 32 / 64 lanes per signal, chunks of 8 / 4 channels
+    (2, 1024, 8, 128, 1.0),
+    (5, 1024, 40, 64, 0.5j),
 ])
 def test_layer_1d(bs, DY, K, N, alpha, tol):
     print("case layer_1d", bs, DY, K, N, alpha, flush=True)
@@ -62,7 +65,8 @@ def test_layer_1d_both_contractions(bs, DY, K, N, alpha, algo, tol, monkeypatch)
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d algo %d" % algo)
 
 
-@pytest.mark.parametrize("DX,DY,nsig", [(128, 128, 3), (256, 128, 2), (128, 256, 2), (256, 256, 2)])
+@pytest.mark.parametrize("DX,DY,nsig", [(128, 128, 3), (256, 128, 2), (128, 256, 2), (256, 256, 2),
+                                        (512, 32, 3), (1024, 48, 2)])
 def test_stride_stages(DX, DY, nsig, tol):
     print("case stride", DX, DY, nsig, flush=True)
     rng = np.random.default_rng(DX + DY)
@@ -91,6 +95,9 @@ def test_stride_stages(DX, DY, nsig, tol):
     (3, 128, 256, 8, 64, 2),
     (2, 256, 128, 24, 128, 2),
     (5, 128, 128, 8, 64, 0),         # auto, more images than one pass of the persistent grid would need
+    (1, 512, 128, 8, 64, 0),         # lengths above 256: auto = three-kernel path
+    (1, 256, 1024, 16, 64, 1),
+    (2, 1024, 512, 8, 64, 0),
 ])
 def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     print("case layer_2d", bs, DX, DY, K, N, algo, flush=True)
@@ -124,9 +131,14 @@ def test_error_codes():
     with pytest.raises(tf.TurboFNOError) as e:
         tf.layer_1d(torch.zeros((8, 1, 2048), dtype=torch.complex64, device="cuda"), W)
     assert e.value.code == 2
+    x2 = torch.zeros((8, 1, 512, 128), dtype=torch.complex64, device="cuda")
+    with pytest.raises(tf.TurboFNOError) as e:                     # whole-image path exists for 128 / 256 only
+        tf.layer_2d(x2, W, algo=2)
+    assert e.value.code == 2
 
 
-@pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128), (1, 128, 16, 64), (5, 256, 8, 64)])
+@pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128), (1, 128, 16, 64), (5, 256, 8, 64),
+                                      (3, 512, 16, 64), (2, 1024, 8, 64)])
 def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     """stages of variants A, B, C: contiguous transforms, cgemm with beta, the two half-fused kernels"""
     print("case variant stages", S, DY, K, N, flush=True)

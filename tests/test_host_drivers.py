@@ -67,7 +67,8 @@ def _run_variant(exe, args):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dim,args", [("1D", (4, 1, 128, 64, 16)), ("1D", (1, 1, 256, 128, 24)),
-                                      ("2D", (1, 128, 256, 64, 16)), ("2D", (2, 256, 128, 64, 8))])
+                                      ("2D", (1, 128, 256, 64, 16)), ("2D", (2, 256, 128, 64, 8)),
+                                      ("1D", (2, 1, 1024, 64, 16)), ("2D", (1, 512, 128, 64, 8))])
 def test_all_variants_agree(dim, args):
     # with TURBOFNO_DIGEST the ten executables reseed rand() per problem and see identical inputs: the staged (A), half-fused (B, C),
     # fully fused (D) and library (E: hipFFT + hipBLAS) sequences must give the same output up to fp32 rounding.

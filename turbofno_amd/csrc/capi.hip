@@ -33,7 +33,8 @@ int log2_exact(long v)
     return l;
 }
 
-bool length_built(int logD) { return logD == 7 || logD == 8; }
+bool length_built(int logD) { return logD >= 7 && logD <= 10; }          // 1D kernels and the X-axis kernels
+bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // whole-image 2D kernels
 
 int check_gemm_dims(long M, int N, int K)
 {
@@ -46,10 +47,17 @@ int check_gemm_dims(long M, int N, int K)
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-int pick_algo(int DX, int DY, int algo)
+// AUTO: the whole-image path runs one persistent block per image, so it needs enough input images (K*bs) to occupy
+// the CUs; below that the three-kernel path spreads an image over many blocks and is faster although it moves 1.5x
+// the bytes. The thresholds are the measured crossovers on MI355X (256 CUs): one image per CU for rows of 256,
+// two / four for the row-128 shapes, whose image kernels stream 64-byte row segments.
+int pick_algo(int bs, int DX, int DY, int K, int algo)
 {
-    (void)DX; (void)DY;   // every built shape has a whole-image kernel
-    return algo != TURBOFNO_2D_AUTO ? algo : TURBOFNO_2D_WHOLE_IMAGE;
+    if (algo != TURBOFNO_2D_AUTO) return algo;
+    if (DX > 256 || DY > 256) return TURBOFNO_2D_THREE_KERNEL;      // an image no longer fits one block's LDS
+    const long images = (long)K * bs;
+    const long need = DY == 256 ? 256 : (DX == 128 ? 512 : 1024);
+    return images >= need ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
 }
 
 }  // namespace
@@ -75,7 +83,7 @@ int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x
     (void)C; (void)beta_re; (void)beta_im;
     if (!x || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and y must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
-    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256, 512, 1024} is built", logDY);
     if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
     hipError_t e = tfno::launch_fused_fft_cgemm_ifft(logDY, M / 64, N, K, (const float2*)x, (const float2*)W, (float2*)y,
                                                      make_float2(alpha_re, alpha_im), algo_1d(), (hipStream_t)stream);
@@ -88,7 +96,7 @@ static int stride_common(bool inverse, int logDX, const void* in, void* out, int
     if (dimX != TURBOFNO_MODES) return fail(TURBOFNO_ERR_INVALID_ARG, "dimX=%d: exactly 64 rows are retained", dimX);
     if (DY <= 0 || DY % 16) return fail(TURBOFNO_ERR_INVALID_ARG, "DY=%d must be a positive multiple of 16", DY);
     if (total <= 0 || total % DY) return fail(TURBOFNO_ERR_INVALID_ARG, "total=%ld must be a positive multiple of DY=%d", total, DY);
-    if (!length_built(logDX)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DX)=%d: only DX in {128, 256} is built", logDX);
+    if (!length_built(logDX)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DX)=%d: only DX in {128, 256, 512, 1024} is built", logDX);
     hipError_t e = inverse ? tfno::launch_ifft_stride(logDX, (const float2*)in, (float2*)out, DY, total / DY, (hipStream_t)stream)
                            : tfno::launch_fft_stride(logDX, (const float2*)in, (float2*)out, DY, total / DY, (hipStream_t)stream);
     return hip_status(e, inverse ? "ifft_stride launch" : "fft_stride launch");
@@ -120,7 +128,7 @@ int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, v
     if (!x || !spec) return fail(TURBOFNO_ERR_INVALID_ARG, "x and spec must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
     const int logDX = log2_exact(DX), logDY = log2_exact(DY);
-    if (!length_built(logDX) || !length_built(logDY))
+    if (!image_length_built(logDX) || !image_length_built(logDY))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
     return hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, (float2*)spec, nimg, (hipStream_t)stream), "fft2d_trunc launch");
 }
@@ -130,7 +138,7 @@ int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, vo
     if (!spec || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "spec and y must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
     const int logDX = log2_exact(DX), logDY = log2_exact(DY);
-    if (!length_built(logDX) || !length_built(logDY))
+    if (!image_length_built(logDX) || !image_length_built(logDY))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
     return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, (const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
 }
@@ -150,7 +158,7 @@ static int stride_DY_common(bool inverse, int logDY, const void* in, void* out, 
 {
     if (!in || !out) return fail(TURBOFNO_ERR_INVALID_ARG, "in and out must be non-null device pointers");
     if (total <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "total=%ld must be positive", total);
-    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256, 512, 1024} is built", logDY);
     hipError_t e = inverse ? tfno::launch_ifft_stride_DY(logDY, (const float2*)in, (float2*)out, total, (hipStream_t)stream)
                            : tfno::launch_fft_stride_DY(logDY, (const float2*)in, (float2*)out, total, (hipStream_t)stream);
     return hip_status(e, inverse ? "ifft_stride_DY launch" : "fft_stride_DY launch");
@@ -173,7 +181,7 @@ int turbofno_fused_fft_cgemm(int logDY, long M, int N, int K, const void* x, con
 {
     if (!x || !W || !C) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and C must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
-    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256, 512, 1024} is built", logDY);
     if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
     return hip_status(tfno::launch_fused_fft_cgemm(logDY, M / 64, N, K, (const float2*)x, (const float2*)W, (float2*)C,
                                                    make_float2(alpha_re, alpha_im), make_float2(beta_re, beta_im),
@@ -186,7 +194,7 @@ int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, co
     (void)C; (void)beta_re; (void)beta_im;
     if (!A || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "A, W and y must be non-null device pointers");
     if (int rc = check_gemm_dims(M, N, K)) return rc;
-    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256} is built", logDY);
+    if (!length_built(logDY)) return fail(TURBOFNO_ERR_UNSUPPORTED, "log2(DY)=%d: only DY in {128, 256, 512, 1024} is built", logDY);
     if (M / 64 > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "M/64=%ld exceeds the grid limit", M / 64);
     return hip_status(tfno::launch_fused_cgemm_ifft(logDY, M / 64, N, K, (const float2*)A, (const float2*)W, (float2*)y,
                                                     make_float2(alpha_re, alpha_im), (hipStream_t)stream),
@@ -196,7 +204,7 @@ int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, co
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
-    if (pick_algo(DX, DY, algo) == TURBOFNO_2D_WHOLE_IMAGE)
+    if (pick_algo(bs, DX, DY, K, algo) == TURBOFNO_2D_WHOLE_IMAGE)
         return align256((size_t)K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
     return align256((size_t)K * bs * 64 * DY * sizeof(float2)) + align256((size_t)N * bs * 64 * DY * sizeof(float2));
 }
@@ -210,10 +218,12 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     if (logDX < 0 || logDY < 0) return fail(TURBOFNO_ERR_INVALID_ARG, "DX=%d, DY=%d must be powers of two", DX, DY);
     if (int rc = check_gemm_dims((long)bs * 64 * 64, N, K)) return rc;
     if (!length_built(logDX) || !length_built(logDY))
-        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256} are built", DX, DY);
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256, 512, 1024} are built", DX, DY);
     if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE)
         return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
-    const int a = pick_algo(DX, DY, algo);
+    if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the whole-image path is built for lengths in {128, 256}", DX, DY);
+    const int a = pick_algo(bs, DX, DY, K, algo);
     const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
     if (!workspace || workspace_bytes < need)
         return fail(TURBOFNO_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need, workspace ? workspace_bytes : (size_t)0);

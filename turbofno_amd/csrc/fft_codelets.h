@@ -274,6 +274,31 @@ TFNO_DEV void inv_pass2(cpx (&e)[16], const cpx (&tw)[16], cpx (&y)[16])
     for (int i = 0; i < 16; ++i) y[i] = e[fft16_slot(i)];
 }
 
+// Lengths 512 and 1024 (L = 32 or 64 lanes per signal). The second pass is no longer a 16- or 8-point transform
+// in registers: after the exchange a lane forms each retained mode as a direct L-term sum, and before the backward
+// exchange each lane builds its 16 first-pass inputs from all 64 modes. Both take their L-point twiddles from the
+// 1024-entry table. `exch` is the group's exchange region as the other lanes left it (pitch-17 rows of first-pass
+// results for the forward direction; the 64 modes in natural order for the backward direction).
+//
+// Forward: mode m = r + 16 c (r = m % 16, c = m / 16 < 4):  X[m] = sum_{tt<L} exch[tt*17 + r] * w_L^(tt c).
+template <int L> TFNO_DEV cpx wide_forward_mode(const cpx* exch, int m)
+{
+    const int r = m & 15, c = m >> 4;
+    cpx acc = make_float2(0.f, 0.f);
+#pragma unroll 8
+    for (int tt = 0; tt < L; ++tt) cfma(acc, exch[tt * 17 + r], kTwiddle1024[(tt * c * (1024 / L)) & 1023]);
+    return acc;
+}
+// Backward: first-pass input r of lane t:  e[r] = sum_{c<4} C[r + 16 c] * conj(w_L^(t c)), C = exch[0..63].
+template <int L> TFNO_DEV void wide_backward_inputs(const cpx* exch, int t, cpx (&e)[16])
+{
+    const cpx w1 = kTwiddle1024[(t * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t * (1024 / L)) & 1023],
+              w3 = kTwiddle1024[(3 * t * (1024 / L)) & 1023];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        e[r] = cadd(cadd(exch[r], cmulc(exch[r + 16], w1)), cadd(cmulc(exch[r + 32], w2), cmulc(exch[r + 48], w3)));
+}
+
 // Orders LDS traffic of one wavefront: everything the wave wrote before is visible to its own
 // lanes after. DS operations of a wave complete in issue order, so no hardware wait is needed
 // beyond what the compiler inserts for the data dependency; this only stops compiler reordering.

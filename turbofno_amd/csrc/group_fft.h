@@ -1,6 +1,6 @@
-// Transforms of one signal by one L-lane group of a wavefront (L = D/16 lanes, 16 samples per lane),
-// built from the register codelets plus one padded LDS exchange that stays inside the wavefront
-// (no block barrier). Shared by the fused 1D kernel and the 2D image kernels.
+// Transforms of one signal by one L-lane group of a wavefront (L = D/16 lanes, 16 samples per lane; L = 8, 16 for
+// lengths 128, 256 and, with direct second-pass sums, L = 32, 64 for lengths 512, 1024), built from the register
+// codelets plus one padded LDS exchange that stays inside the wavefront (no block barrier). Shared by the fused 1D kernel and the 2D image kernels.
 #pragma once
 #include "fft_codelets.h"
 
@@ -32,6 +32,9 @@ TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&o
 #pragma unroll
         for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
         dft16_first4<-1>(u, out);                       // out[s] = X[t + 16 s]
+    } else if constexpr (L >= 32) {
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) out[mm] = wide_forward_mode<L>(exch, t + L * mm);
     } else {
         cpx u0[8], u1[8], o0[4], o1[4];
 #pragma unroll
@@ -59,7 +62,10 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
 {
     constexpr int L = Geo1D<LOGDY>::L;
     wave_lds_fence();
-    if constexpr (L == 16) {
+    if constexpr (L >= 32) {
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
+    } else if constexpr (L == 16) {
         cpx h[16];
         dft16_pad4<+1>(c, h);
 #pragma unroll
@@ -75,8 +81,12 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
     }
     wave_lds_fence();
     cpx e[16];
+    if constexpr (L >= 32) {
+        wide_backward_inputs<L>(exch, t, e);
+    } else {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+        for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+    }
     inv_pass2(e, tw, y);
 }
 
@@ -87,6 +97,7 @@ TFNO_DEV void group_backward_lds(const cpx (&c)[Geo1D<LOGD>::MM], const cpx* twr
 {
     constexpr int L = Geo1D<LOGD>::L;
     wave_lds_fence();
+    static_assert(L <= 16, "the whole-image kernels are built for lengths 128 and 256");
     if constexpr (L == 16) {
         cpx h[16];
         dft16_pad4<+1>(c, h);

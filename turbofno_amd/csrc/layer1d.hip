@@ -307,6 +307,8 @@ static hipError_t dispatch_fused_1d(int logDY, long S, int N, int K, const float
     switch (logDY) {
     case 7: return launch_fused_1d<7, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
     case 8: return launch_fused_1d<8, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
+    case 9: return launch_fused_1d<9, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
+    case 10: return launch_fused_1d<10, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -370,6 +372,8 @@ hipError_t launch_fft_stride_DY(int logDY, const float2* in, float2* out, long n
     switch (logDY) {
     case 7: return launch_stride_DY_t<7, false>(in, out, nsig, stream);
     case 8: return launch_stride_DY_t<8, false>(in, out, nsig, stream);
+    case 9: return launch_stride_DY_t<9, false>(in, out, nsig, stream);
+    case 10: return launch_stride_DY_t<10, false>(in, out, nsig, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -379,6 +383,8 @@ hipError_t launch_ifft_stride_DY(int logDY, const float2* in, float2* out, long 
     switch (logDY) {
     case 7: return launch_stride_DY_t<7, true>(in, out, nsig, stream);
     case 8: return launch_stride_DY_t<8, true>(in, out, nsig, stream);
+    case 9: return launch_stride_DY_t<9, true>(in, out, nsig, stream);
+    case 10: return launch_stride_DY_t<10, true>(in, out, nsig, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -43,7 +43,19 @@ __global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void fft_stride_kernel(c
     for (int r = 0; r < 16; ++r) lds[(t * 17 + r) * 16 + yl] = g[r];
     __syncthreads();
     float2* dst = out + sig * 64 * DY + y;
-    if constexpr (L == 16) {
+    if constexpr (L >= 32) {
+        // lengths 512 / 1024: each retained row m = t + L*mm is a direct L-term sum over the first-pass results
+        // (the same arithmetic as wide_forward_mode, on this kernel's [t][r][yl] exchange layout)
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) {
+            const int m = t + L * mm, r = m & 15, c = m >> 4;
+            cpx acc = make_float2(0.f, 0.f);
+#pragma unroll 8
+            for (int tt = 0; tt < L; ++tt)
+                cfma(acc, lds[(tt * 17 + r) * 16 + yl], kTwiddle1024[(tt * c * (1024 / L)) & 1023]);
+            dst[(long)m * DY] = acc;
+        }
+    } else if constexpr (L == 16) {
         cpx u[16], o[4];
 #pragma unroll
         for (int tt = 0; tt < 16; ++tt) u[tt] = lds[(tt * 17 + t) * 16 + yl];
@@ -82,7 +94,10 @@ __global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void ifft_stride_kernel(
     cpx tw[16];
     load_lane_twiddles<LOGDX>(t, tw);
     const float2* src = in + sig * 64 * DY + y;
-    if constexpr (L == 16) {
+    if constexpr (L >= 32) {
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) lds[(t + L * mm) * 16 + yl] = src[(long)(t + L * mm) * DY];
+    } else if constexpr (L == 16) {
         cpx c[4], h[16];
 #pragma unroll
         for (int s = 0; s < 4; ++s) c[s] = src[(long)(t + 16 * s) * DY];
@@ -106,8 +121,18 @@ __global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void ifft_stride_kernel(
     }
     __syncthreads();
     cpx e[16], yv[16];
+    if constexpr (L >= 32) {
+        // first-pass input r of row group t from the 64 retained rows (wide_backward_inputs on this layout)
+        const cpx w1 = kTwiddle1024[(t * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t * (1024 / L)) & 1023],
+                  w3 = kTwiddle1024[(3 * t * (1024 / L)) & 1023];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * 16 + yl];
+        for (int r = 0; r < 16; ++r)
+            e[r] = cadd(cadd(lds[r * 16 + yl], cmulc(lds[(r + 16) * 16 + yl], w1)),
+                        cadd(cmulc(lds[(r + 32) * 16 + yl], w2), cmulc(lds[(r + 48) * 16 + yl], w3)));
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * 16 + yl];
+    }
     inv_pass2(e, tw, yv);
     float2* dst = out + (sig * DX + t) * DY + y;
 #pragma unroll
@@ -121,6 +146,16 @@ static hipError_t launch_stride_t(const float2* in, float2* out, int DY, long ns
     long blocks = nsig * DY / 16;
     if (blocks <= 0 || blocks > 0x7fffffffL) return hipErrorInvalidValue;
     dim3 grid((unsigned)blocks, 1, 1), block(G::THREADS, 1, 1);
+    if constexpr (G::LDS_BYTES > 64 * 1024) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            const void* fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX>)
+                                     : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX>);
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
+            if (e != hipSuccess) return e;
+            attr_set = true;
+        }
+    }
     if (INVERSE) hipLaunchKernelGGL(ifft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
     else hipLaunchKernelGGL(fft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
     return hipGetLastError();
@@ -131,6 +166,8 @@ hipError_t launch_fft_stride(int logDX, const float2* in, float2* out, int DY, l
     switch (logDX) {
     case 7: return launch_stride_t<7, false>(in, out, DY, nsig, stream);
     case 8: return launch_stride_t<8, false>(in, out, DY, nsig, stream);
+    case 9: return launch_stride_t<9, false>(in, out, DY, nsig, stream);
+    case 10: return launch_stride_t<10, false>(in, out, DY, nsig, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -140,6 +177,8 @@ hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, 
     switch (logDX) {
     case 7: return launch_stride_t<7, true>(in, out, DY, nsig, stream);
     case 8: return launch_stride_t<8, true>(in, out, DY, nsig, stream);
+    case 9: return launch_stride_t<9, true>(in, out, DY, nsig, stream);
+    case 10: return launch_stride_t<10, true>(in, out, DY, nsig, stream);
     default: return hipErrorInvalidValue;
     }
 }
