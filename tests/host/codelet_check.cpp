@@ -149,6 +149,69 @@ template <int LOGD> static double check_wide(bool backward)
     return std::sqrt(num / den);
 }
 
+// rows of 128 handled by 16 lanes, two rows of 8 samples per lane (the whole-image kernels' row pass for DY = 128):
+// lane t holds samples t + 16 i of row A and row B, after the exchange lane t = r + 8 h finishes row h, modes r + 8 c.
+static double check_rows128(bool backward)
+{
+    constexpr int D = 128;
+    std::vector<cpx> exch(16 * 17);
+    cpx tw[16][8];
+    for (int t = 0; t < 16; ++t)
+        for (int r = 0; r < 8; ++r) tw[t][r] = kTwiddle1024[((t * r) << 3) & 1023];
+    double num = 0, den = 0;
+    if (!backward) {
+        std::vector<cpx> x(2 * D);
+        for (auto& v : x) v = make_float2((float)frand(), (float)frand());
+        for (int t = 0; t < 16; ++t) {
+            cpx a[8], b[8];
+            for (int i = 0; i < 8; ++i) { a[i] = x[t + 16 * i]; b[i] = x[D + t + 16 * i]; }
+            fft8<-1>(a);
+            fft8<-1>(b);
+            for (int r = 0; r < 8; ++r) { exch[t * 17 + r] = cmul(a[r], tw[t][r]); exch[t * 17 + 8 + r] = cmul(b[r], tw[t][r]); }
+        }
+        for (int t = 0; t < 16; ++t) {
+            cpx u[16], out[8];
+            for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
+            dft16_first8<-1>(u, out);
+            const int row = t >> 3, r = t & 7;
+            for (int c = 0; c < 8; ++c) {
+                const int m = r + 8 * c;
+                zd acc = 0;
+                for (int j = 0; j < D; ++j)
+                    acc += zd(x[row * D + j].x, x[row * D + j].y) * std::polar(1.0, -2.0 * M_PI * ((long)j * m % D) / D);
+                num += std::norm(acc - zd(out[c].x, out[c].y));
+                den += std::norm(acc);
+            }
+        }
+    } else {
+        std::vector<cpx> C(2 * 64), y(2 * D);
+        for (auto& v : C) v = make_float2((float)frand(), (float)frand());
+        for (int t = 0; t < 16; ++t) {
+            const int row = t >> 3, r = t & 7;
+            cpx c[8], h[16];
+            for (int k = 0; k < 8; ++k) c[k] = C[row * 64 + r + 8 * k];
+            dft16_pad8<+1>(c, h);
+            for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+        }
+        for (int t = 0; t < 16; ++t) {
+            cpx a[8], b[8];
+            for (int r = 0; r < 8; ++r) { a[r] = cmulc(exch[t * 17 + r], tw[t][r]); b[r] = cmulc(exch[t * 17 + 8 + r], tw[t][r]); }
+            fft8<+1>(a);
+            fft8<+1>(b);
+            for (int i = 0; i < 8; ++i) { y[t + 16 * i] = a[i]; y[D + t + 16 * i] = b[i]; }
+        }
+        for (int row = 0; row < 2; ++row)
+            for (int j = 0; j < D; ++j) {
+                zd acc = 0;
+                for (int m = 0; m < 64; ++m)
+                    acc += zd(C[row * 64 + m].x, C[row * 64 + m].y) * std::polar(1.0, 2.0 * M_PI * ((long)j * m % D) / D);
+                num += std::norm(acc - zd(y[row * D + j].x, y[row * D + j].y));
+                den += std::norm(acc);
+            }
+    }
+    return std::sqrt(num / den);
+}
+
 int main()
 {
     srand(12345);
@@ -162,6 +225,9 @@ int main()
         if (!(v < 5e-7)) { printf("FAIL\n"); return 1; }
     for (double v : w)
         if (!(v < 5e-7)) { printf("FAIL\n"); return 1; }
+    const double p0 = check_rows128(false), p1 = check_rows128(true);
+    printf("rows128  : fwd %.3e bwd %.3e\n", p0, p1);
+    if (!(p0 < 5e-7) || !(p1 < 5e-7)) { printf("FAIL\n"); return 1; }
     printf("OK\n");
     return 0;
 }

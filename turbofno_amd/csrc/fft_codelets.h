@@ -188,6 +188,48 @@ template <int DIR> TFNO_DEV void dft8_pad4(const cpx (&c)[4], cpx (&h)[8])
     }
 }
 
+// 8-point FFT in registers, natural order in and out.
+template <int DIR> TFNO_DEV void fft8(cpx (&v)[8])
+{
+    // i = i0 + 2 i1:  B_i0[rho] = sum_i1 v[i0 + 2 i1] w4^(i1 rho);  F[rho + 4 sigma] = B_0[rho] + (-1)^sigma w8^rho B_1[rho]
+    radix4<DIR>(v[0], v[2], v[4], v[6]);
+    radix4<DIR>(v[1], v[3], v[5], v[7]);
+    const cpx w0 = v[1], w1 = mul_w16<DIR, 2>(v[3]), w2 = mul_w16<DIR, 4>(v[5]), w3 = mul_w16<DIR, 6>(v[7]);
+    const cpx b0 = v[0], b1 = v[2], b2 = v[4], b3 = v[6];
+    v[0] = cadd(b0, w0); v[1] = cadd(b1, w1); v[2] = cadd(b2, w2); v[3] = cadd(b3, w3);
+    v[4] = csub(b0, w0); v[5] = csub(b1, w1); v[6] = csub(b2, w2); v[7] = csub(b3, w3);
+}
+
+// First eight bins of a 16-point DFT:  out[c] = sum_{t<16} u[t] w16^(t c), c = 0..7.
+template <int DIR> TFNO_DEV void dft16_first8(const cpx (&u)[16], cpx (&out)[8])
+{
+    // t = 2 t1 + t0:  out[c] = E[c] + w16^c O[c], E / O = 8-point transforms of the even / odd samples
+    cpx e[8], o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { e[i] = u[2 * i]; o[i] = u[2 * i + 1]; }
+    fft8<DIR>(e);
+    fft8<DIR>(o);
+    out[0] = cadd(e[0], o[0]);                    out[1] = cadd(e[1], mul_w16<DIR, 1>(o[1]));
+    out[2] = cadd(e[2], mul_w16<DIR, 2>(o[2]));   out[3] = cadd(e[3], mul_w16<DIR, 3>(o[3]));
+    out[4] = cadd(e[4], mul_w16<DIR, 4>(o[4]));   out[5] = cadd(e[5], mul_w16<DIR, 5>(o[5]));
+    out[6] = cadd(e[6], mul_w16<DIR, 6>(o[6]));   out[7] = cadd(e[7], mul_w16<DIR, 7>(o[7]));
+}
+
+// 16-point DFT of an 8-element input padded with 8 zeros:  h[t] = sum_{c<8} c[c] w16^(t c), t = 0..15.
+template <int DIR> TFNO_DEV void dft16_pad8(const cpx (&c)[8], cpx (&h)[16])
+{
+    // c = 2 s + c0:  h[j] = H0[j] + w16^j H1[j],  h[j + 8] = H0[j] - w16^j H1[j],  H = 8-point pad transforms of even / odd inputs
+    cpx ce[4], co[4], h0[8], h1[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { ce[i] = c[2 * i]; co[i] = c[2 * i + 1]; }
+    dft8_pad4<DIR>(ce, h0);
+    dft8_pad4<DIR>(co, h1);
+    const cpx w[8] = { h1[0], mul_w16<DIR, 1>(h1[1]), mul_w16<DIR, 2>(h1[2]), mul_w16<DIR, 3>(h1[3]),
+                       mul_w16<DIR, 4>(h1[4]), mul_w16<DIR, 5>(h1[5]), mul_w16<DIR, 6>(h1[6]), mul_w16<DIR, 7>(h1[7]) };
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { h[j] = cadd(h0[j], w[j]); h[j + 8] = csub(h0[j], w[j]); }
+}
+
 // Per-lane inter-pass twiddles  tw[r] = w_D^(t r), r = 0..15, for lane t of an L-lane group (D = 16 L).
 template <int LOGD> TFNO_DEV void load_lane_twiddles(int t, cpx (&tw)[16])
 {
@@ -204,7 +246,7 @@ constexpr int kTwLdsSize = 16 * kTwLdsPitch;   // complex elements
 #ifndef TFNO_HOST_CHECK
 template <int LOGD> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
 {
-    for (int e = tid; e < 16 * ((1 << LOGD) / 16); e += nthreads) {
+    for (int e = tid; e < 256; e += nthreads) {      // all 16 lane rows (groups of fewer lanes use the first ones)
         const int t = e >> 4, r = e & 15;
         tab[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
     }

@@ -119,4 +119,48 @@ TFNO_DEV void group_backward_lds(const cpx (&c)[Geo1D<LOGD>::MM], const cpx* twr
     inv_pass2_lds(e, twrow, y);
 }
 
+// Rows of 128 in the whole-image kernels: a 16-lane group owns TWO rows, lane t holds samples t + 16 i (i < 8) of
+// each, so a group still moves 128 contiguous bytes per load or store. The first pass is a pair of 8-point FFTs;
+// after the exchange lane t = r + 8 h finishes row h: modes r + 8 c, c < 8. Twiddles w_128^(t r) come from the lane's
+// row of the LDS table.
+#ifndef TFNO_HOST_CHECK
+// g[0..7] / g[8..15]: first-pass results of row A / row B, already twiddled. On return out[c] = mode (t & 7) + 8 c
+// of row (t >> 3).
+TFNO_DEV void rows128_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&out)[8])
+{
+    wave_lds_fence();
+#pragma unroll
+    for (int j = 0; j < 16; ++j) exch[t * 17 + j] = g[j];
+    wave_lds_fence();
+    cpx u[16];
+#pragma unroll
+    for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
+    dft16_first8<-1>(u, out);
+}
+
+// c[k] = mode (t & 7) + 8 k of row (t >> 3). On return y[i] / y[8 + i] = sample t + 16 i of row A / row B.
+TFNO_DEV void rows128_backward(const cpx (&c)[8], const cpx* twrow, cpx* exch, int t, cpx (&y)[16])
+{
+    cpx h[16];
+    dft16_pad8<+1>(c, h);
+    wave_lds_fence();
+#pragma unroll
+    for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+    wave_lds_fence();
+    cpx a[8], b[8];
+    a[0] = exch[t * 17];
+    b[0] = exch[t * 17 + 8];
+#pragma unroll
+    for (int r = 1; r < 8; ++r) {
+        const cpx w = twrow[r];
+        a[r] = cmulc(exch[t * 17 + r], w);
+        b[r] = cmulc(exch[t * 17 + 8 + r], w);
+    }
+    fft8<+1>(a);
+    fft8<+1>(b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { y[i] = a[i]; y[8 + i] = b[i]; }
+}
+#endif
+
 }  // namespace tfno

@@ -25,26 +25,40 @@ constexpr int TPITCH = 66;                       // row pitch (complex) of the D
 constexpr int EXCH_ELEMS = 1024 * 17;            // exchange regions of all lane groups of a 1024-thread block
 
 // Geometry of the whole-image kernels for a DX x DY image (DX rows of DY contiguous samples).
+// Rows of 256: a 16-lane group owns one row (16 samples per lane). Rows of 128 ("paired"): a 16-lane group owns
+// two rows, 8 samples per lane each, so that a group still covers 128 contiguous bytes per access.
 template <int LOGX, int LOGY> struct Geo2D {
     static constexpr int DX = 1 << LOGX, DY = 1 << LOGY;
-    static constexpr int LX = DX / 16, LY = DY / 16;          // lanes per column / per row transform
-    static constexpr int GY = 1024 / LY;                      // rows transformed concurrently
-    static constexpr int ITY = DX / GY;                       // row passes per image
-    static constexpr int MMY = 64 / LY, MMX = 64 / LX;        // modes per lane after a row / column transform
+    static constexpr bool PAIRED = LOGY == 7;
+    static constexpr int LX = DX / 16, LY = 16;               // lanes per column / per row-pass group
+    static constexpr int GY = 1024 / LY;                      // lane groups of the row pass
+    static constexpr int RPP = PAIRED ? 2 * GY : GY;          // rows per pass
+    static constexpr int ITY = DX / RPP;                      // row passes per image
+    static constexpr int MMY = PAIRED ? 8 : 4;                // modes per lane after one row pass
+    static constexpr int MMX = 64 / LX;                       // modes per lane after the column pass
     static constexpr int COLT = 64 * LX;                      // threads that take part in the column pass
     static constexpr int TILE = DX * TPITCH;
     static constexpr int LDS_MAIN = EXCH_ELEMS > TILE ? EXCH_ELEMS : TILE;   // exchange regions alias the tile
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(LDS_MAIN + 2 * kTwLdsSize);
+    static_assert(LOGY == 7 || LOGY == 8, "rows of 128 or 256");
     static_assert(ITY >= 1 && COLT <= 1024, "unsupported image shape");
+    // element offset of the lane's i-th sample from its first one
+    static __device__ __forceinline__ constexpr int sample_off(int i) { return PAIRED ? (i & 7) * 16 + (i >> 3) * (4 * DY) : 16 * i; }
 };
 
-// Row (within one pass of GY rows) handled by lane group g. The 32/LY groups that share an LDS cycle (one half
-// wavefront) get rows LY/2 apart, so that their pitch-66 tile accesses fall on disjoint banks.
-template <int LY> __device__ __forceinline__ int row_in_pass(int g)
+// First row (within one pass) of lane group g. The two groups that share an LDS cycle (one half wavefront) must
+// hit disjoint banks of the pitch-66 tile, i.e. sit 8 rows apart (4 rows = 16 banks).
+//   rows of 256: one row per group; groups 2j, 2j+1 get rows 8 apart.
+//   rows of 128: group g owns rows a and a + 4 (lanes 0-7 / 8-15 finish one each: 16 banks apart), a enumerating the
+//   rows with bit 2 clear; groups 2j, 2j+1 again 8 rows apart.
+template <bool PAIRED> __device__ __forceinline__ int first_row_in_pass(int g)
 {
-    constexpr int GH = 32 / LY, HS = LY / 2;     // groups per half wavefront, row spacing between them
-    const int jh = g % GH, rest = g / GH;
-    return jh * HS + (rest % HS) + (rest / HS) * 16;
+    const int jh = g & 1, rest = g >> 1;
+    if constexpr (!PAIRED) return jh * 8 + (rest % 8) + (rest / 8) * 16;
+    else {
+        const int s = jh * 4 + (rest % 4) + (rest / 4) * 8;    // pair index, partner groups 4 apart
+        return (s & 3) + 8 * (s >> 2);
+    }
 }
 }  // namespace
 
@@ -76,15 +90,18 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
     __syncthreads();
 
-    const int row0 = row_in_pass<LY>(gy);
+    const int row0 = first_row_in_pass<G::PAIRED>(gy);
+    // row the lane finishes after the exchange, and its first mode (paired rows: lanes 8-15 take the second row)
+    const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;
+    const int tq = G::PAIRED ? (ty & 7) : ty;
     // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
     const unsigned lane_off = (unsigned)(row0 * DY + ty);
     // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
     // next kernel re-reads, out of L2 / Infinity Cache
     auto issue = [&](cpx (&dst)[16], long img, int it, unsigned off) {
-        const float2* base = x + (img * DX + GY * it) * (long)DY;
+        const float2* base = x + (img * DX + G::RPP * it) * (long)DY;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + (unsigned)(LY * i)]);
+        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + (unsigned)G::sample_off(i)]);
     };
 
     long img = blockIdx.x;
@@ -96,24 +113,48 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
         const bool more = img + gridDim.x < nimg;
         const long pre = more ? img + gridDim.x : 0;
         const unsigned pre_off = more ? lane_off : (unsigned)ty;
-        // pass 1: rows (along Y). T[it][mm] = mode q = ty + LY mm of row row0 + GY it
+        // pass 1: rows (along Y). T[it][mm] = mode tq + 16 mm (paired rows: tq + 8 mm) of row trow + RPP it
         cpx T[ITY][MMY];
 #pragma unroll
         for (int it = 0; it < ITY; ++it) {
-            cpx bb[16], gg[16];
-            fft16_stage1<-1>(v, bb);
-            // v is dead after the first radix-4 stage: its registers become the landing zone of the next row;
-            // the last pass already fetches the next image's first row
-            if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
-            else issue(v, pre, 0, pre_off);
-            fwd_pass1_lds_finish(bb, twrow_y, gg);
-            group_forward_finish<LOGY>(gg, exch_y, ty, T[it]);
+            if constexpr (!G::PAIRED) {
+                cpx bb[16], gg[16];
+                fft16_stage1<-1>(v, bb);
+                // v is dead after the first radix-4 stage: its registers become the landing zone of the next row;
+                // the last pass already fetches the next image's first row
+                if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
+                else issue(v, pre, 0, pre_off);
+                fwd_pass1_lds_finish(bb, twrow_y, gg);
+                group_forward_finish<8>(gg, exch_y, ty, T[it]);
+            } else {
+                cpx gg[16], b8[8];
+                {
+                    cpx a8[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) { a8[i] = v[i]; b8[i] = v[8 + i]; }
+                    fft8<-1>(a8);
+                    fft8<-1>(b8);
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) gg[r] = a8[r];
+                }
+                if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
+                else issue(v, pre, 0, pre_off);
+                gg[8] = b8[0];
+#pragma unroll
+                for (int r = 1; r < 8; ++r) {
+                    const cpx w = twrow_y[r];
+                    gg[r] = cmul(gg[r], w);
+                    gg[8 + r] = cmul(b8[r], w);
+                }
+                rows128_forward_finish(gg, exch_y, ty, T[it]);
+            }
         }
         __syncthreads();
 #pragma unroll
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
-            for (int mm = 0; mm < MMY; ++mm) lds[(row0 + GY * it) * TPITCH + ty + LY * mm] = T[it][mm];
+            for (int mm = 0; mm < MMY; ++mm)
+                lds[(trow + G::RPP * it) * TPITCH + tq + (G::PAIRED ? 8 : 16) * mm] = T[it][mm];
         __syncthreads();
         // pass 2: columns (along X); group gx owns column q = gx, lane tx holds rows tx + LX i
         cpx c[16];
@@ -158,7 +199,9 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
     __syncthreads();
 
-    const int row0 = row_in_pass<LY>(gy);
+    const int row0 = first_row_in_pass<G::PAIRED>(gy);
+    const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;      // row whose modes the lane takes from the tile
+    const int tq = G::PAIRED ? (ty & 7) : ty;
     const unsigned lane_off = (unsigned)(row0 * DY + ty);
     const bool col_thread = tid < G::COLT;
 
@@ -189,7 +232,8 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 #pragma unroll
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
-            for (int mm = 0; mm < MMY; ++mm) cc[it][mm] = lds[(row0 + GY * it) * TPITCH + ty + LY * mm];
+            for (int mm = 0; mm < MMY; ++mm)
+                cc[it][mm] = lds[(trow + G::RPP * it) * TPITCH + tq + (G::PAIRED ? 8 : 16) * mm];
         __syncthreads();
         // pass 2: rows (q -> y), coalesced row stores.
         // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
@@ -197,10 +241,11 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 #pragma unroll
         for (int it = 0; it < ITY; ++it) {
             cpx yv[16];
-            group_backward_lds<LOGY>(cc[it], twrow_y, exch_y, ty, yv);
-            float2* dst = y + (img * DX + GY * it) * (long)DY;   // uniform base + lane offset + immediates
+            if constexpr (G::PAIRED) rows128_backward(cc[it], twrow_y, exch_y, ty, yv);
+            else group_backward_lds<8>(cc[it], twrow_y, exch_y, ty, yv);
+            float2* dst = y + (img * DX + G::RPP * it) * (long)DY;   // uniform base + lane offset + immediates
 #pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + LY * i, yv[i]);
+            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + G::sample_off(i), yv[i]);
         }
     }
 }
