@@ -177,3 +177,28 @@ def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     torch.cuda.synchronize()
     ref = oracle.ifft_pad_contig(oracle.cgemm(A32, W, alpha).reshape(N, S, 64), DY)
     check(y, ref, tol, "fused_cgemm_ifft")
+
+
+@pytest.mark.parametrize("DX,DY", [(256, 256), (128, 256), (256, 128), (128, 128)])
+def test_image_stage_entry_points(DX, DY, tol):
+    """turbofno_fft2d_trunc / turbofno_ifft2d_pad on their own, through the documented order of the 4096 retained
+    modes: element mm*(64*LX) + q*LX + t holds mode (p = t + LX*mm, q), LX = DX/16"""
+    print("case image stages", DX, DY, flush=True)
+    nimg, LX = 3, DX // 16
+    rng = np.random.default_rng(DX * 3 + DY)
+    x = (rng.uniform(-1, 1, (nimg, DX, DY)) + 1j * rng.uniform(-1, 1, (nimg, DX, DY))).astype(np.complex64)
+    e = np.arange(4096)
+    mm, q, t = e // (64 * LX), (e % (64 * LX)) // LX, e % LX
+    p = t + LX * mm
+    spec = torch.empty((nimg, 4096), dtype=torch.complex64, device="cuda")
+    tf.fft2d_trunc(dev(x), spec)
+    torch.cuda.synchronize()
+    full = np.fft.fft2(x.astype(np.complex128), axes=(1, 2))
+    check(spec, full[:, p, q], tol, "fft2d_trunc")
+    modes = (rng.uniform(-1, 1, (nimg, 64, 64)) + 1j * rng.uniform(-1, 1, (nimg, 64, 64))).astype(np.complex64)
+    y = torch.empty((nimg, DX, DY), dtype=torch.complex64, device="cuda")
+    tf.ifft2d_pad(dev(modes[:, p, q]), y)
+    torch.cuda.synchronize()
+    padded = np.zeros((nimg, DX, DY), dtype=np.complex128)
+    padded[:, :64, :64] = modes
+    check(y, np.fft.ifft2(padded, axes=(1, 2)) * (DX * DY), tol, "ifft2d_pad")

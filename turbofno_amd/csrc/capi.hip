@@ -49,15 +49,15 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // AUTO: the whole-image path runs one persistent block per image, so it needs enough input images (K*bs) to occupy
 // the CUs; below that the three-kernel path spreads an image over many blocks and is faster although it moves 1.5x
-// the bytes. The thresholds are the measured crossovers on MI355X (256 CUs): one image per CU for rows of 256,
-// two / four for the row-128 shapes, whose image kernels stream 64-byte row segments.
+// the bytes. Measured crossover on MI355X (256 CUs): one input image per CU, and for images smaller than 256 x 256
+// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner).
 int pick_algo(int bs, int DX, int DY, int K, int algo)
 {
     if (algo != TURBOFNO_2D_AUTO) return algo;
     if (DX > 256 || DY > 256) return TURBOFNO_2D_THREE_KERNEL;      // an image no longer fits one block's LDS
     const long images = (long)K * bs;
-    const long need = DY == 256 ? 256 : (DX == 128 ? 512 : 1024);
-    return images >= need ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
+    const bool big = DX == 256 && DY == 256;
+    return (images >= 256 && (big || bs >= 8)) ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
 }
 
 }  // namespace
