@@ -20,8 +20,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--bs", type=int, default=16)
     ap.add_argument("--algo", type=int, default=0, help="0 auto, 1 three-kernel pipeline, 2 whole-image")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -87,13 +87,13 @@ def main():
             ev[s][2].record(); tf.ifft2d_pad(cspec, y)
             ev[s][3].record()
         torch.cuda.synchronize()
-        names = ["fft2d_trunc_256", "cgemm_modes", "ifft2d_pad_256"]
+        names = ["fft2d_trunc", "cgemm_modes", "ifft2d_pad"]
         for i, nme in enumerate(names):
             stages[nme] = float(np.mean([ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(args.steps)]))
         # dominant kernel = the longer of the two image kernels; its algorithmic bytes = one pass over
         # its side of the layer (input read once / output written once)
-        dom = max(("fft2d_trunc_256", "ifft2d_pad_256"), key=lambda k: stages[k])
-        dom_bytes = img_bytes * (K if dom == "fft2d_trunc_256" else N)
+        dom = max(("fft2d_trunc", "ifft2d_pad"), key=lambda k: stages[k])
+        dom_bytes = img_bytes * (K if dom == "fft2d_trunc" else N)
         achieved = dom_bytes / (stages[dom] * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
@@ -145,6 +145,19 @@ def main():
         except Exception as exc:  # pragma: no cover - informational only
             comparators["unfused_rocfft_rocblas_ms"] = "failed: %s" % type(exc).__name__
 
+    # ---- the 1D large-hidden case (bs=64, DY=256, K=N=128): where the contraction runs on the matrix cores -------
+    large_hidden = None
+    if not args.no_comparators:
+        x1_h, W1_h = workloads.smooth_1d(0x5EED + 3, 64, 256, 128, 128)
+        x1, W1 = torch.from_numpy(x1_h).to(dev), torch.from_numpy(W1_h).to(dev)
+        y1 = torch.empty((128, 64, 256), dtype=torch.complex64, device=dev)
+        t1d = timed(lambda: tf.layer_1d(x1, W1, y=y1), 50)
+        b1d = 8 * 64 * 256 * (128 + 128) + 8 * 128 * 128
+        f1d = 8.0 * (64 * 64) * 128 * 128                      # real flops of the complex contraction
+        large_hidden = {"workload": "1D bs=64 DY=256 K=128 N=128", "ms": round(t1d, 4),
+                        "GBps": round(b1d / (t1d * 1e-3) / 1e9, 1), "hbm_frac": round(b1d / (t1d * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "contraction_TFLOPs": round(f1d / (t1d * 1e-3) / 1e12, 2), "fp32_mfma_peak_TFLOPs": 157.3}
+
     # ---- CPU baseline: fp32 OpenMP restatement of the library baseline, bounded sample -------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -174,7 +187,7 @@ def main():
         "layer_algorithmic_bytes": layer_bytes, "layer_GBps": round(layer_gbs, 1),
         "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall_ms, 4),
         "stage_ms": {k: round(v, 4) for k, v in stages.items()},
-        "roofline": roofline, "cpu_baseline": cpu, "comparators": comparators,
+        "roofline": roofline, "cpu_baseline": cpu, "comparators": comparators, "large_hidden_1d": large_hidden,
     }
     print(json.dumps(out))
 
