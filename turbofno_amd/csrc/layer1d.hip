@@ -145,7 +145,8 @@ template <int LOGDY> struct GeoMfma1D {
     static constexpr int PA = 80, PC = 72;                    // pitches (complex) of sA and sC
     static constexpr int EXCH = L * 17;
     static constexpr int REGION0 = KC * EXCH > KC * PA ? KC * EXCH : KC * PA;              // exchange | sA
-    static constexpr int REGION1 = KC * 128 > 64 * PC ? KC * 128 : 64 * PC;                // W' | sC   (complex)
+    static constexpr int WTILE = (KC / 4) * kWGroup / 2;                                   // W' tile in complex units
+    static constexpr int REGION1 = WTILE > 64 * PC ? WTILE : 64 * PC;                      // W' | sC   (complex)
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
 };
 
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
     constexpr int DY = 1 << LOGDY, L = G::L, MM = G::MM, KC = G::KC, PA = G::PA, PC = G::PC;
     extern __shared__ float2 lds[];
     float2* sA = lds;                                          // [KC][PA]; aliases the exchange regions
-    float* sW = reinterpret_cast<float*>(lds + G::REGION0);    // [(k/4)][(k&3)>>1][n' 128][k&1][c]
+    float* sW = reinterpret_cast<float*>(lds + G::REGION0);    // W' tile, layout of kWGroup / kWHalf
     float2* sC = lds + G::REGION0;                             // [64][PC]; aliases sW after the K loop
 
     const int tid = threadIdx.x;
@@ -212,18 +213,18 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
             const int idx = tid + u * G::THREADS;
             const int k = idx % KC, n = idx / KC;
             const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
-            float* dstw = &sW[(k >> 2) * 1024 + ((k & 3) >> 1) * 512 + (2 * n) * 4 + (k & 1) * 2];
+            float* dstw = &sW[(k >> 2) * kWGroup + ((k & 3) >> 1) * kWHalf + (2 * n) * 4 + (k & 1) * 2];
             *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
             *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
         }
         __syncthreads();
         const float2* arow = sA + kq * PA + mt * 16 + col;
-        const float* wrow = sW + (kq >> 1) * 512 + (nt0 * 16 + col) * 4 + (kq & 1) * 2;
+        const float* wrow = sW + (kq >> 1) * kWHalf + (nt0 * 16 + col) * 4 + (kq & 1) * 2;
         for (int kg = 0; kg < kn / 4; ++kg) {
             const float2 b = arow[kg * 4 * PA];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float2 a = *reinterpret_cast<const float2*>(wrow + kg * 1024 + i * 64);
+                const float2 a = *reinterpret_cast<const float2*>(wrow + kg * kWGroup + i * 64);
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[i], 0, 0, 0);
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[i], 0, 0, 0);
             }

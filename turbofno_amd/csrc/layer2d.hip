@@ -267,7 +267,6 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
-constexpr int GEMM_WGROUP = 1024;   // floats per group of 4 channels in the W tile: [(k&3)>>1][n' (128)][k&1][c]
 constexpr int GEMM_THREADS = 1024;  // 16 waves x 16 m
 constexpr int GEMM_MBLOCK = 256;    // m per block
 
@@ -275,10 +274,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
                                                                    const float2* __restrict__ W, float2* __restrict__ C,
                                                                    long Mtot, int N, int K, float2 alpha, float2 beta)
 {
-    // sW[(k/4)*1024 + ((k&3)>>1)*512 + n'*4 + (k&1)*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:
+    // sW[(k/4)*kWGroup + ((k&3)>>1)*kWHalf + n'*4 + (k&1)*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:
     // {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1. In one operand read (16 n' x 4 channels) lanes 0-31 cover 256
     // contiguous bytes in lane order pairs and lanes 32-63 the next 256: no bank conflicts.
-    __shared__ float sW[(GEMM_KC / 4) * GEMM_WGROUP];
+    extern __shared__ float sW[];                     // (GEMM_KC / 4) * kWGroup floats
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.y * 64;
     switch (wave >> 2) {                      // waves w, w+4, w+8, w+12 share a SIMD
@@ -310,7 +309,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
             bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         __syncthreads();
         // W tile: lanes run along k, the contiguous direction of W[k + n*K], so a wave reads 512 contiguous bytes
-        // (the LDS stores then collide on banks, but there are only eight of them per lane)
         constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
         float2 wv[WPT];
 #pragma unroll
@@ -324,7 +322,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
             const int idx = tid + u * GEMM_THREADS;
             const int k = idx % GEMM_KC, n = idx / GEMM_KC;
             const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
-            float* dstw = &sW[(k >> 2) * GEMM_WGROUP + ((k & 3) >> 1) * 512 + (2 * n) * 4 + (k & 1) * 2];
+            float* dstw = &sW[(k >> 2) * kWGroup + ((k & 3) >> 1) * kWHalf + (2 * n) * 4 + (k & 1) * 2];
             *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
             *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
         }
@@ -334,10 +332,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
         // stored at once, so its stores drain under the matrix work of the following tiles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const float* wrow = &sW[(kq >> 1) * 512 + (t * 16 + col) * 4 + (kq & 1) * 2];
+            const float* wrow = &sW[(kq >> 1) * kWHalf + (t * 16 + col) * 4 + (kq & 1) * 2];
 #pragma unroll
             for (int g = 0; g < GEMM_KC / 4; ++g) {
-                const float2 a = *reinterpret_cast<const float2*>(wrow + g * GEMM_WGROUP);
+                const float2 a = *reinterpret_cast<const float2*>(wrow + g * kWGroup);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, bv[g].x, acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, bv[g].y, acc[t], 0, 0, 0);
             }
@@ -418,7 +416,15 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
 {
     if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
-    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), 0, stream, A, W, C, Mtot, N, K, alpha, beta);
+    constexpr size_t lds_bytes = sizeof(float) * (GEMM_KC / 4) * kWGroup;      // 66,048 B: above the static limit
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(cgemm_modes_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
     return hipGetLastError();
 }
 
