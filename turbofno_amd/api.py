@@ -139,7 +139,7 @@ def layer_2d(x, W, y=None, alpha=1.0 + 0j, workspace=None, algo=0):
 
 
 def fft2d_trunc(x, spec):
-    """x: [nimg][256][256] -> spec: [nimg][4096] (retained 64 x 64 modes, kernel-private order)."""
+    """x: [nimg][DX][DY], DX, DY in {128, 256} -> spec: [nimg][4096] (retained 64 x 64 modes, kernel-private order)."""
     nimg = x.numel() // (x.shape[-1] * x.shape[-2])
     _check(lib().turbofno_fft2d_trunc(x.shape[-2], x.shape[-1], _dev_c64(x, "x"), _dev_c64(spec, "spec"), nimg,
                                       _stream()))
@@ -147,7 +147,7 @@ def fft2d_trunc(x, spec):
 
 
 def ifft2d_pad(spec, y):
-    """spec: [nimg][4096] -> y: [nimg][256][256]."""
+    """spec: [nimg][4096] -> y: [nimg][DX][DY]."""
     nimg = y.numel() // (y.shape[-1] * y.shape[-2])
     _check(lib().turbofno_ifft2d_pad(y.shape[-2], y.shape[-1], _dev_c64(spec, "spec"), _dev_c64(y, "y"), nimg,
                                      _stream()))

@@ -1,6 +1,7 @@
 // Internal launcher declarations shared between the kernel translation units and the C ABI.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 
 namespace tfno {
 
@@ -13,8 +14,23 @@ namespace tfno {
 constexpr int kWHalf = 516;
 constexpr int kWGroup = 1032;
 
-// compute units of the current device (cached)
+// compute units of the current device (cached per device)
 int cu_count();
+
+// Kernels with more than 64 KiB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize raised once per device.
+// `done` is the kernel's own bit mask of devices already served (one static per launcher); safe from several threads:
+// a second caller at worst repeats the idempotent call.
+inline hipError_t allow_dynamic_lds(const void* kernel, size_t bytes, std::atomic<unsigned long long>& done)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
 
 // 1D fused layer / Y stage of the three-kernel 2D pipeline. S = number of signals per channel.
 // algo: 0 = chosen by size, 1 = SIMT contraction, 2 = contraction on the matrix cores.

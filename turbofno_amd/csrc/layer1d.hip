@@ -319,13 +319,10 @@ static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const
                                     hipStream_t stream)
 {
     using G = GeoMfma1D<LOGDY>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static std::atomic<unsigned long long> served;
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY>), G::LDS_BYTES, served);
+        e != hipSuccess)
+        return e;
     hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY>), dim3((unsigned)S, (unsigned)(N / 64)), dim3(G::THREADS),
                        G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();

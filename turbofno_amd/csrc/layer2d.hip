@@ -357,28 +357,24 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
 
 int cu_count()
 {
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
-        else cus = 256;
-    }
-    return cus;
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    int v = cached[dev & 63].load(std::memory_order_relaxed);
+    if (v > 0) return v;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cached[dev & 63].store(v, std::memory_order_relaxed);
+    return v;
 }
 
 template <int LOGX, int LOGY>
 static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, long nimg, hipStream_t stream)
 {
     using G = Geo2D<LOGX, LOGY>;
-    static bool attr_set[2] = { false, false };
+    static std::atomic<unsigned long long> served[2];
     const void* fn = inverse ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY>)
                              : reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>);
-    if (!attr_set[inverse]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set[inverse] = true;
-    }
+    if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse]); e != hipSuccess) return e;
     // persistent blocks: at most as many as fit at once (LDS allows one or two 1024-thread blocks per CU,
     // the thread count exactly one)
     const long blocks = nimg < cu_count() ? nimg : cu_count();
@@ -417,13 +413,9 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
     if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     constexpr size_t lds_bytes = sizeof(float) * (GEMM_KC / 4) * kWGroup;      // 66,048 B: above the static limit
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(cgemm_modes_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static std::atomic<unsigned long long> served;
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes_kernel), lds_bytes, served); e != hipSuccess)
+        return e;
     hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
     return hipGetLastError();
 }

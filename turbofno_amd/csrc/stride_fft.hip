@@ -147,14 +147,10 @@ static hipError_t launch_stride_t(const float2* in, float2* out, int DY, long ns
     if (blocks <= 0 || blocks > 0x7fffffffL) return hipErrorInvalidValue;
     dim3 grid((unsigned)blocks, 1, 1), block(G::THREADS, 1, 1);
     if constexpr (G::LDS_BYTES > 64 * 1024) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            const void* fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX>)
-                                     : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX>);
-            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
-            if (e != hipSuccess) return e;
-            attr_set = true;
-        }
+        static std::atomic<unsigned long long> served;
+        const void* fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX>)
+                                 : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX>);
+        if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served); e != hipSuccess) return e;
     }
     if (INVERSE) hipLaunchKernelGGL(ifft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
     else hipLaunchKernelGGL(fft_stride_kernel<LOGDX>, grid, block, G::LDS_BYTES, stream, in, out, DY);
