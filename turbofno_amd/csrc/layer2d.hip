@@ -17,6 +17,7 @@
 // lanes coincide, every access is contiguous per wavefront) and the GEMM is oblivious to it.
 #include "group_fft.h"
 #include "kernels.h"
+#include <type_traits>
 
 namespace tfno {
 
@@ -270,6 +271,10 @@ constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
 constexpr int GEMM_THREADS = 1024;  // 16 waves x 16 m
 constexpr int GEMM_MBLOCK = 256;    // m per block
 
+// NG = channel groups of four per chunk that can hold data: 16 in general; 4, 8 or 12 for K <= 16, 32, 48, where the
+// single chunk then does no loads and no matrix work on zero padding. A template parameter so that the loops stay
+// unrolled and branch free.
+template <int NG>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
                                                                    const float2* __restrict__ W, float2* __restrict__ C,
                                                                    long Mtot, int N, int K, float2 alpha, float2 beta)
@@ -303,9 +308,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
         const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;   // multiple of 8 (caller contract)
         const bool last = kc + GEMM_KC >= K;
         // the wave's whole A strip of this chunk: lane (kq, col) holds channels kc + 4 g + kq, g = 0..15
-        float2 bv[GEMM_KC / 4];
+        float2 bv[NG];
 #pragma unroll
-        for (int g = 0; g < GEMM_KC / 4; ++g)
+        for (int g = 0; g < NG; ++g)
             bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         __syncthreads();
         // W tile: lanes run along k, the contiguous direction of W[k + n*K], so a wave reads 512 contiguous bytes
@@ -334,7 +339,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
         for (int t = 0; t < 8; ++t) {
             const float* wrow = &sW[(kq >> 1) * kWHalf + (t * 16 + col) * 4 + (kq & 1) * 2];
 #pragma unroll
-            for (int g = 0; g < GEMM_KC / 4; ++g) {
+            for (int g = 0; g < NG; ++g) {
                 const float2 a = *reinterpret_cast<const float2*>(wrow + g * kWGroup);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, bv[g].x, acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, bv[g].y, acc[t], 0, 0, 0);
@@ -413,11 +418,19 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
     if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     constexpr size_t lds_bytes = sizeof(float) * (GEMM_KC / 4) * kWGroup;      // 66,048 B: above the static limit
-    static std::atomic<unsigned long long> served;
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes_kernel), lds_bytes, served); e != hipSuccess)
-        return e;
-    hipLaunchKernelGGL(cgemm_modes_kernel, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
-    return hipGetLastError();
+    auto launch = [&](auto ng_const) -> hipError_t {
+        constexpr int NG = decltype(ng_const)::value;
+        static std::atomic<unsigned long long> served;
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes_kernel<NG>), lds_bytes, served);
+            e != hipSuccess)
+            return e;
+        hipLaunchKernelGGL(cgemm_modes_kernel<NG>, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
+        return hipGetLastError();
+    };
+    if (K <= 16) return launch(std::integral_constant<int, 4>{});
+    if (K <= 32) return launch(std::integral_constant<int, 8>{});
+    if (K <= 48) return launch(std::integral_constant<int, 12>{});
+    return launch(std::integral_constant<int, 16>{});
 }
 
 }  // namespace tfno
