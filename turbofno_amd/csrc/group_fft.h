@@ -13,8 +13,10 @@ template <int LOGDY> struct Geo1D {
     static constexpr int MM = 64 / L;        // modes owned per lane   (m = lane + L*mm)
     static constexpr int NN = 64 / GROUPS;   // output channels per group (n = g + GROUPS*jn)
     static constexpr int EXCH = L * 17;      // complex per group exchange region
-    static constexpr int SA_PITCH = 64;
-    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * 64 + GROUPS * EXCH);
+    // pitches (complex) of the spectra tile sA[kk][m] and the weight tile sW[kk][n] of the fused kernel: rows of sA are
+    // written by neighbouring lane groups at once (80: half the banks apart), rows of sW by consecutive lanes (65)
+    static constexpr int SA_PITCH = 80, SW_PITCH = 65;
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * SW_PITCH + GROUPS * EXCH);
 };
 
 // second half of the forward transform: exchange of the twiddled first-pass results g[] inside the

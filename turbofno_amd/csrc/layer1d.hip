@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
     extern __shared__ float2 lds[];
     float2* sA = lds;                                  // [GROUPS][64]   truncated spectra of the K chunk
     float2* sW = sA + GROUPS * G::SA_PITCH;            // [GROUPS][64]   W chunk, sW[kk][n]
-    float2* exch_all = sW + GROUPS * 64;
+    float2* exch_all = sW + GROUPS * G::SW_PITCH;
 
     const int tid = threadIdx.x;
     const int g = tid / L, t = tid % L;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
             int kk = idx % GROUPS, n = idx / GROUPS;
             float2 w = make_float2(0.f, 0.f);
             if (kc + kk < K) w = W[(kc + kk) + (long)(n0 + n) * K];
-            sW[kk * 64 + n] = w;
+            sW[kk * G::SW_PITCH + n] = w;
         }
         __syncthreads();
 #pragma unroll 4
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 #pragma unroll
             for (int i = 0; i < MM; ++i) a[i] = sA[kk * G::SA_PITCH + t + L * i];
 #pragma unroll
-            for (int j = 0; j < NN; ++j) b[j] = sW[kk * 64 + g + GROUPS * j];
+            for (int j = 0; j < NN; ++j) b[j] = sW[kk * G::SW_PITCH + g + GROUPS * j];
 #pragma unroll
             for (int i = 0; i < MM; ++i)
 #pragma unroll
