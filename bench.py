@@ -173,7 +173,11 @@ def main():
             oracle.cpu_baseline_layer_2d(xs, W_h, 1.0, cores)
             best = min(best, time.perf_counter() - t)
             reps += 1
+        t = time.perf_counter()
+        oracle.cpu_baseline_layer_2d(xs, W_h, 1.0, 1)
+        one_core_ms = (time.perf_counter() - t) * 1e3 * (bs / sample_bs)
         cpu = {"value": round(best * 1e3 * (bs / sample_bs), 2), "unit": "ms/layer", "cores": cores, "kind": "port",
+               "one_core_ms_per_layer": round(one_core_ms, 1),
                "sample": "bs=%d of the same workload (K=N=64, 256x256), best of %d runs, scaled x%d to bs=%d"
                          % (sample_bs, reps, bs // sample_bs, bs)}
 

@@ -148,6 +148,7 @@ int main(int argc, char** argv)
         else
             printf("1D_%c, bs=%-4d, dimX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", TURBOFNO_VARIANT, p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
         fflush(stdout);
+        if (getenv("TURBOFNO_STATS")) print_iteration_stats(launch, ntest);
         HIP_RT_CALL(hipEventDestroy(t_begin));
         HIP_RT_CALL(hipEventDestroy(t_end));
         HIP_RT_CALL(hipFree(dx)); HIP_RT_CALL(hipFree(dw)); HIP_RT_CALL(hipFree(dy));

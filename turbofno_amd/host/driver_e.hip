@@ -142,6 +142,7 @@ int main(int argc, char** argv)
         else
             printf("1D_E, bs=%-4d, dimX=%-4d, DY=%-4d, N=%-4d, K=%-4d, TIME=%8.3fms\n", p.bs, p.dx, p.dy, p.n, p.k, elapsed_time);
         fflush(stdout);
+        if (getenv("TURBOFNO_STATS")) print_iteration_stats(launch, ntest);
         CHECK_FFT(hipfftDestroy(plan_in));
         CHECK_FFT(hipfftDestroy(plan_out));
         HIP_RT_CALL(hipEventDestroy(t_begin)); HIP_RT_CALL(hipEventDestroy(t_end));

@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <cstdio>
+#include <algorithm>
 #include <cstdlib>
 #include <map>
 #include <string>
@@ -24,6 +25,27 @@ void generate_random_vector(float* target, long n);
 // generating each problem's inputs: every variant of a problem then sees the same inputs and must print the same
 // digest up to fp32 rounding.
 void print_output_digest(const void* device_y, size_t complex_elems);
+
+// With TURBOFNO_STATS set the drivers add, after the reference-format result line, one line
+// "  stats: min=<ms> median=<ms> max=<ms> over <n> iterations" from per-iteration events around the same launches
+// (the result line itself stays the mean over launch + device synchronise, as in the reference).
+template <class Launch> void print_iteration_stats(Launch&& launch, int n)
+{
+    std::vector<hipEvent_t> ev(2 * (size_t)n);
+    for (auto& e : ev) (void)hipEventCreate(&e);
+    for (int i = 0; i < n; ++i) {
+        (void)hipEventRecord(ev[2 * i]);
+        launch();
+        (void)hipEventRecord(ev[2 * i + 1]);
+        (void)hipDeviceSynchronize();
+    }
+    std::vector<float> ms(n);
+    for (int i = 0; i < n; ++i) (void)hipEventElapsedTime(&ms[i], ev[2 * i], ev[2 * i + 1]);
+    std::sort(ms.begin(), ms.end());
+    printf("  stats: min=%.4fms median=%.4fms max=%.4fms over %d iterations\n", ms.front(), ms[n / 2], ms.back(), n);
+    fflush(stdout);
+    for (auto& e : ev) (void)hipEventDestroy(e);
+}
 
 #define HIP_RT_CALL(call)                                                                                    \
     do {                                                                                                     \
