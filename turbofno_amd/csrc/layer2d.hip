@@ -76,7 +76,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
                                                            int nimg)
 {
     using G = Geo2D<LOGX, LOGY>;
-    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, GY = G::GY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
+    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x;
     const int gy = tid / LY, ty = tid % LY;            // row pass: group and lane
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
                                                           int nimg)
 {
     using G = Geo2D<LOGX, LOGY>;
-    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, GY = G::GY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
+    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x;
     const int gy = tid / LY, ty = tid % LY;
