@@ -33,7 +33,7 @@ inline hipError_t allow_dynamic_lds(const void* kernel, size_t bytes, std::atomi
 }
 
 // 1D fused layer / Y stage of the three-kernel 2D pipeline. S = number of signals per channel.
-// algo: 0 = chosen by size, 1 = SIMT contraction, 2 = contraction on the matrix cores.
+// algo: 0 = chosen by size, 1 = SIMT contraction, 2 / 3 = contraction on the matrix cores (512- / 256-thread blocks).
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream);
 

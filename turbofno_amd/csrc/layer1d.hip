@@ -126,8 +126,8 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 // arithmetic (K >= one chunk). Same operands, grid (S, N/64) and block-traverses-K schedule as the kernel above;
 // 512 threads = 8 waves:
 //   * a chunk is KC = 512/L channels (32 for DY=256, 64 for DY=128): every L-lane group transforms one channel and
-//     leaves its 64 modes in sA[k][m]; the loads of the next chunk are issued as soon as the first pass has consumed
-//     the registers, so they travel under the exchange, the W tile build and the matrix work;
+//     leaves its 64 modes in sA[k][m]; two chunks of loads are in flight per group (a buffer is refilled as soon as the
+//     first pass has consumed it), so they travel under the exchanges, the W tile builds and the matrix work;
 //   * C'[n'][m] += W'[n'][k'] A'[k'][m] is the 4-real form of the complex product on v_mfma_f32_16x16x4_f32:
 //     n' = (n, re|im) 128 rows, m 64 columns = 8 x 4 tiles, four per wave (one m tile, four n' tiles), so one read of
 //     A from LDS feeds eight matrix instructions. W' (alpha folded in) uses the conflict-free LDS order of
@@ -138,9 +138,10 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 // sC aliases the W' tile.
 typedef float floatx4_1d __attribute__((ext_vector_type(4)));
 
-template <int LOGDY> struct GeoMfma1D {
+template <int LOGDY, int THREADS_> struct GeoMfma1D {
     static constexpr int L = Geo1D<LOGDY>::L, MM = 64 / L;
-    static constexpr int THREADS = 512;
+    static constexpr int THREADS = THREADS_;                  // 512: one block per CU; 256: two (LDS 72 KiB each)
+    static constexpr int NTW = 32 / (THREADS / 64);           // 16x16 tiles per wave: one m tile x NTW n' tiles
     static constexpr int KC = THREADS / L;                    // channels per chunk = lane groups per block
     static constexpr int PA = 80, PC = 72;                    // pitches (complex) of sA and sC
     static constexpr int EXCH = L * 17;
@@ -150,12 +151,13 @@ template <int LOGDY> struct GeoMfma1D {
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
 };
 
-template <int LOGDY>
-__global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
-                                                                  const float2* __restrict__ W, float2* __restrict__ y,
-                                                                  float2 alpha)
+template <int LOGDY, int THREADS>
+__global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
+                                                                      const float2* __restrict__ W, float2* __restrict__ y,
+                                                                      float2 alpha)
 {
-    using G = GeoMfma1D<LOGDY>;
+    using G = GeoMfma1D<LOGDY, THREADS>;
+    constexpr int NTW = G::NTW;
     constexpr int DY = 1 << LOGDY, L = G::L, MM = G::MM, KC = G::KC, PA = G::PA, PC = G::PC;
     extern __shared__ float2 lds[];
     float2* sA = lds;                                          // [KC][PA]; aliases the exchange regions
@@ -165,7 +167,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
     const int tid = threadIdx.x;
     const int g = tid / L, t = tid % L;                        // transform role: lane group = channel of the chunk
     const int wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;   // matrix role
-    const int mt = wave & 3, nt0 = (wave >> 2) * 4;            // m tile, first of four n' tiles
+    const int mt = wave & 3, nt0 = (wave >> 2) * NTW;          // m tile, first of the wave's NTW n' tiles
     const long s = blockIdx.x;
     const int n0 = blockIdx.y * 64;
     float2* exch = lds + g * G::EXCH;
@@ -173,19 +175,21 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
     cpx tw[16];
     load_lane_twiddles<LOGDY>(t, tw);
 
-    floatx4_1d acc[4];
+    floatx4_1d acc[NTW];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
+    for (int i = 0; i < NTW; ++i) acc[i] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
 
     auto issue = [&](cpx (&dst)[16], int k) {
         const float2* src = x + ((long)k * S + s) * DY + t;
 #pragma unroll
         for (int i = 0; i < 16; ++i) dst[i] = src[L * i];
     };
-    cpx v[16];
-    if (g < K) issue(v, g);
+    // two chunks of loads in flight per lane group: buffer b receives chunk c + 2 as soon as chunk c has left it
+    cpx v0[16], v1[16];
+    if (g < K) issue(v0, g);
+    if (KC + g < K) issue(v1, KC + g);
 
-    for (int kc = 0; kc < K; kc += KC) {
+    auto chunk = [&](cpx (&v)[16], int kc) {
         const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
         // W chunk: lanes run along k, the contiguous direction of W[k + n*K]
         constexpr int WPT = KC * 64 / G::THREADS;
@@ -200,7 +204,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
         if (g < kn) {
             cpx gg[16];
             fwd_pass1(v, tw, gg);
-            if (kc + KC + g < K) issue(v, kc + KC + g);        // next chunk's channel of this group
+            if (kc + 2 * KC + g < K) issue(v, kc + 2 * KC + g);    // this group's channel two chunks ahead
             group_forward_finish<LOGDY>(gg, exch, t, out);
         }
         __syncthreads();                                       // all exchanges done: sA may overwrite them
@@ -223,18 +227,22 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_kernel(int S, int N, 
         for (int kg = 0; kg < kn / 4; ++kg) {
             const float2 b = arow[kg * 4 * PA];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < NTW; ++i) {
                 const float2 a = *reinterpret_cast<const float2*>(wrow + kg * kWGroup + i * 64);
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[i], 0, 0, 0);
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[i], 0, 0, 0);
             }
         }
         __syncthreads();                                       // sA / sW are free again (next chunk, or sC below)
+    };
+    for (int kc = 0; kc < K; kc += 2 * KC) {
+        chunk(v0, kc);
+        if (kc + KC < K) chunk(v1, kc + KC);
     }
 
     // D[row = 4 kq + v][col] of tile i: n' = 16 (nt0 + i) + 4 kq + v = 2 n + c'  ->  n = 8 (nt0 + i) + 2 kq + (v >> 1)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NTW; ++i) {
         const int n = 8 * (nt0 + i) + 2 * kq;
         sC[n * PC + mt * 16 + col] = make_float2(acc[i][0], acc[i][1]);
         sC[(n + 1) * PC + mt * 16 + col] = make_float2(acc[i][2], acc[i][3]);
@@ -314,31 +322,40 @@ static hipError_t dispatch_fused_1d(int logDY, long S, int N, int K, const float
     }
 }
 
-template <int LOGDY>
+template <int LOGDY, int THREADS>
 static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
                                     hipStream_t stream)
 {
-    using G = GeoMfma1D<LOGDY>;
+    using G = GeoMfma1D<LOGDY, THREADS>;
     static std::atomic<unsigned long long> served;
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY>), G::LDS_BYTES, served);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY, THREADS>),
+                                         G::LDS_BYTES, served);
         e != hipSuccess)
         return e;
-    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY>), dim3((unsigned)S, (unsigned)(N / 64)), dim3(G::THREADS),
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS>), dim3((unsigned)S, (unsigned)(N / 64)), dim3(THREADS),
                        G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();
 }
 
-// algo: 0 = by size (matrix cores once K fills a chunk of the 512-thread kernel), 1 = SIMT kernel, 2 = matrix cores
+// algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
-    // by size: the matrix-core kernel needs K to fill a chunk, and it keeps one 8-wave block per CU, so it wins while
-    // every block has a CU to itself (measured crossover: about one block per CU); beyond that the SIMT kernel's
-    // three blocks per CU hide more latency
-    const bool fills = (logDY == 8 && K >= 32) || (logDY == 7 && K >= 64);
-    const bool mfma = algo == 2 || (algo == 0 && fills && S * (N / 64) <= cu_count());
-    if (mfma && logDY == 8) return launch_fused_mfma<8>(S, N, K, x, W, y, alpha, stream);
-    if (mfma && logDY == 7) return launch_fused_mfma<7>(S, N, K, x, W, y, alpha, stream);
+    // by size (measured crossovers on MI355X):
+    //  * while every block has a CU to itself and K fills a 512-thread chunk: matrix cores, 8 waves per block (the
+    //    shortest chain of latencies);
+    //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two per CU - the SIMT kernel is bound by its
+    //    vector instructions there, more than half of which are the contraction;
+    //  * otherwise the SIMT kernel (three blocks per CU, no idle lanes in short chunks).
+    int pick = algo;
+    if (pick == 0) {
+        const bool fills = (logDY == 8 && K >= 32) || (logDY == 7 && K >= 64);
+        pick = (fills && S * (N / 64) <= cu_count()) ? 2 : (K >= 64 ? 3 : 1);
+    }
+    if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream);
     return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream);
 }
 
