@@ -143,16 +143,22 @@ template <int LOGDY, int THREADS_> struct GeoMfma1D {
     static constexpr int THREADS = THREADS_;                  // 512: one block per CU; 256: two (LDS 72 KiB each)
     static constexpr int NTW = 32 / (THREADS / 64);           // 16x16 tiles per wave: one m tile x NTW n' tiles
     static constexpr int KC = THREADS / L;                    // channels per chunk = lane groups per block
-    static constexpr int PA = 80, PC = 72;                    // pitches (complex) of sA and sC
+    // compact: sC shares the exchange regions too and the twiddles move to LDS: 53 KiB and 168 registers, three blocks
+    // per CU. Only for DY = 256: at DY = 128 (8 modes per lane) the register limit costs more in spills than it gains.
+    static constexpr bool COMPACT = THREADS_ == 256 && LOGDY == 8;
+    static constexpr int PA = 80, PC = COMPACT ? 66 : 72;     // pitches (complex) of sA and sC
     static constexpr int EXCH = L * 17;
     static constexpr int REGION0 = KC * EXCH > KC * PA ? KC * EXCH : KC * PA;              // exchange | sA
     static constexpr int WTILE = (KC / 4) * kWGroup / 2;                                   // W' tile in complex units
-    static constexpr int REGION1 = WTILE > 64 * PC ? WTILE : 64 * PC;                      // W' | sC   (complex)
-    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
+    static constexpr int REGION1 = COMPACT ? WTILE : (WTILE > 64 * PC ? WTILE : 64 * PC);  // W' | sC   (complex)
+    static_assert(!COMPACT || 64 * PC <= REGION0, "sC must fit the exchange regions");
+    static constexpr int TWTAB = COMPACT ? kTwLdsSize : 0;    // compact: twiddles in LDS instead of 30 registers
+    static constexpr int DEPTH = COMPACT ? 1 : 2;             // chunks of loads in flight per lane group
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1 + TWTAB);
 };
 
 template <int LOGDY, int THREADS>
-__global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
+__global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                       const float2* __restrict__ W, float2* __restrict__ y,
                                                                       float2 alpha)
 {
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
     extern __shared__ float2 lds[];
     float2* sA = lds;                                          // [KC][PA]; aliases the exchange regions
     float* sW = reinterpret_cast<float*>(lds + G::REGION0);    // W' tile, layout of kWGroup / kWHalf
-    float2* sC = lds + G::REGION0;                             // [64][PC]; aliases sW after the K loop
+    float2* sC = G::COMPACT ? lds : lds + G::REGION0;          // [64][PC]; aliases sW (or sA) after the K loop
 
     const int tid = threadIdx.x;
     const int g = tid / L, t = tid % L;                        // transform role: lane group = channel of the chunk
@@ -173,7 +179,13 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
     float2* exch = lds + g * G::EXCH;
 
     cpx tw[16];
-    load_lane_twiddles<LOGDY>(t, tw);
+    const float2* twrow = lds + G::REGION0 + G::REGION1 + t * kTwLdsPitch;
+    if constexpr (G::COMPACT) {
+        fill_lds_twiddles<LOGDY>(lds + G::REGION0 + G::REGION1, tid, THREADS);
+        __syncthreads();
+    } else {
+        load_lane_twiddles<LOGDY>(t, tw);
+    }
 
     floatx4_1d acc[NTW];
 #pragma unroll
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
     // two chunks of loads in flight per lane group: buffer b receives chunk c + 2 as soon as chunk c has left it
     cpx v0[16], v1[16];
     if (g < K) issue(v0, g);
-    if (KC + g < K) issue(v1, KC + g);
+    if (G::DEPTH == 2 && KC + g < K) issue(v1, KC + g);
 
     auto chunk = [&](cpx (&v)[16], int kc) {
         const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
@@ -203,8 +215,9 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
         cpx out[MM];
         if (g < kn) {
             cpx gg[16];
-            fwd_pass1(v, tw, gg);
-            if (kc + 2 * KC + g < K) issue(v, kc + 2 * KC + g);    // this group's channel two chunks ahead
+            if constexpr (G::COMPACT) fwd_pass1_lds(v, twrow, gg);
+            else fwd_pass1(v, tw, gg);
+            if (kc + G::DEPTH * KC + g < K) issue(v, kc + G::DEPTH * KC + g);    // this group's channel DEPTH chunks ahead
             group_forward_finish<LOGDY>(gg, exch, t, out);
         }
         __syncthreads();                                       // all exchanges done: sA may overwrite them
@@ -235,9 +248,9 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
         }
         __syncthreads();                                       // sA / sW are free again (next chunk, or sC below)
     };
-    for (int kc = 0; kc < K; kc += 2 * KC) {
+    for (int kc = 0; kc < K; kc += G::DEPTH * KC) {
         chunk(v0, kc);
-        if (kc + KC < K) chunk(v1, kc + KC);
+        if (G::DEPTH == 2 && kc + KC < K) chunk(v1, kc + KC);
     }
 
     // D[row = 4 kq + v][col] of tile i: n' = 16 (nt0 + i) + 4 kq + v = 2 n + c'  ->  n = 8 (nt0 + i) + 2 kq + (v >> 1)
@@ -248,13 +261,20 @@ __global__ __launch_bounds__(THREADS) void fused_fft_mfma_ifft_kernel(int S, int
         sC[(n + 1) * PC + mt * 16 + col] = make_float2(acc[i][2], acc[i][3]);
     }
     __syncthreads();
+    // every pass takes its modes before the first backward transform: in the compact layout the exchange regions
+    // overlay sC
+    cpx c[64 / KC][MM];
+#pragma unroll
+    for (int pass = 0; pass < 64 / KC; ++pass)
+#pragma unroll
+        for (int a = 0; a < MM; ++a) c[pass][a] = sC[(g + KC * pass) * PC + t + L * a];
+    if constexpr (G::COMPACT) __syncthreads();
 #pragma unroll
     for (int pass = 0; pass < 64 / KC; ++pass) {
         const int n = g + KC * pass;
-        cpx c[MM], yv[16];
-#pragma unroll
-        for (int a = 0; a < MM; ++a) c[a] = sC[n * PC + t + L * a];
-        group_backward<LOGDY>(c, tw, exch, t, yv);
+        cpx yv[16];
+        if constexpr (G::COMPACT) group_backward_lds<LOGDY>(c[pass], twrow, exch, t, yv);
+        else group_backward<LOGDY>(c[pass], tw, exch, t, yv);
         float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
 #pragma unroll
         for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
@@ -344,8 +364,8 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     // by size (measured crossovers on MI355X):
     //  * while every block has a CU to itself and K fills a 512-thread chunk: matrix cores, 8 waves per block (the
     //    shortest chain of latencies);
-    //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two per CU - the SIMT kernel is bound by its
-    //    vector instructions there, more than half of which are the contraction;
+    //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
+    //    its vector instructions there, more than half of which are the contraction;
     //  * otherwise the SIMT kernel (three blocks per CU, no idle lanes in short chunks).
     int pick = algo;
     if (pick == 0) {
