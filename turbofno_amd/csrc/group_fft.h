@@ -141,7 +141,8 @@ TFNO_DEV void rows128_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (
 }
 
 // c[k] = mode (t & 7) + 8 k of row (t >> 3). On return y[i] / y[8 + i] = sample t + 16 i of row A / row B.
-TFNO_DEV void rows128_backward(const cpx (&c)[8], const cpx* twrow, cpx* exch, int t, cpx (&y)[16])
+template <class TW>   // twrow[r] = w_128^(t r), r < 8: a row of the LDS table or a register array
+TFNO_DEV void rows128_backward(const cpx (&c)[8], const TW& twrow, cpx* exch, int t, cpx (&y)[16])
 {
     cpx h[16];
     dft16_pad8<+1>(c, h);
@@ -162,6 +163,29 @@ TFNO_DEV void rows128_backward(const cpx (&c)[8], const cpx* twrow, cpx* exch, i
     fft8<+1>(b);
 #pragma unroll
     for (int i = 0; i < 8; ++i) { y[i] = a[i]; y[8 + i] = b[i]; }
+}
+
+// The same pairing for the 1D kernels, with the twiddles in registers (tw[r] = w_128^(t r), t < 16): a 16-lane group
+// transforms two signals; v[0..7] / v[8..15] are samples t + 16 i of signal A / signal B. On return out[c] is mode
+// (t & 7) + 8 c of signal (t >> 3): the lane-to-mode mapping of an 8-lane group per signal, so callers index their
+// tiles as for L = 8 and only the loads and stores change to 128-byte segments.
+TFNO_DEV void pair128_forward(const cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t, cpx (&out)[8])
+{
+    cpx a[8], b[8], g[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { a[i] = v[i]; b[i] = v[8 + i]; }
+    fft8<-1>(a);
+    fft8<-1>(b);
+    g[0] = a[0];
+    g[8] = b[0];
+#pragma unroll
+    for (int r = 1; r < 8; ++r) { g[r] = cmul(a[r], tw[r]); g[8 + r] = cmul(b[r], tw[r]); }
+    rows128_forward_finish(g, exch, t, out);
+}
+// c[k] = mode (t & 7) + 8 k of signal (t >> 3); on return y[i] / y[8 + i] = sample t + 16 i of signal A / signal B.
+TFNO_DEV void pair128_backward(const cpx (&c)[8], const cpx (&tw)[16], cpx* exch, int t, cpx (&y)[16])
+{
+    rows128_backward(c, tw, exch, t, y);
 }
 #endif
 

@@ -37,10 +37,14 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
     const long s = blockIdx.x;
     const int n0 = blockIdx.y * 64;
     const long M = 64L * S;
-    float2* exch = exch_all + g * G::EXCH;
+    // signals of 128 samples are transformed in pairs by 16-lane groups (128-byte accesses): lane t16 of pair g/2 holds
+    // samples t16 + 16 i of both signals, and ends up with the modes an 8-lane group would give lane (g, t)
+    constexpr bool PAIR = LOGDY == 7;
+    const int t16 = tid % 16, gpair = (tid / 16) * 2;
+    float2* exch = PAIR ? exch_all + (tid / 16) * (2 * G::EXCH) : exch_all + g * G::EXCH;
 
     cpx tw[16];
-    load_lane_twiddles<LOGDY>(t, tw);
+    load_lane_twiddles<LOGDY>(PAIR ? t16 : t, tw);
 
     cpx acc[MM][NN];
 #pragma unroll
@@ -53,11 +57,18 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
             const int k = kc + g;
             cpx out[MM];
             if (k < K) {
-                const float2* src = x + ((long)k * S + s) * DY + t;
                 cpx v[16];
+                if constexpr (PAIR) {
+                    const float2* src = x + ((long)(kc + gpair) * S + s) * DY + t16;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[i] = src[L * i];
-                group_forward<LOGDY>(v, tw, exch, t, out);
+                    for (int i = 0; i < 8; ++i) { v[i] = src[16 * i]; v[8 + i] = src[(long)S * DY + 16 * i]; }
+                    pair128_forward(v, tw, exch, t16, out);
+                } else {
+                    const float2* src = x + ((long)k * S + s) * DY + t;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[i] = src[L * i];
+                    group_forward<LOGDY>(v, tw, exch, t, out);
+                }
             } else {
 #pragma unroll
                 for (int a = 0; a < MM; ++a) out[a] = make_float2(0.f, 0.f);
@@ -106,10 +117,17 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
             cpx c[MM], yv[16];
 #pragma unroll
             for (int i = 0; i < MM; ++i) c[i] = cmul(acc[i][j], alpha);
-            group_backward<LOGDY>(c, tw, exch, t, yv);
-            float2* dst = y + ((long)n * S + s) * DY + t;
+            if constexpr (PAIR) {
+                pair128_backward(c, tw, exch, t16, yv);
+                float2* dst = y + ((long)(n0 + gpair + GROUPS * j) * S + s) * DY + t16;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+                for (int i = 0; i < 8; ++i) { dst[16 * i] = yv[i]; dst[(long)S * DY + 16 * i] = yv[8 + i]; }
+            } else {
+                group_backward<LOGDY>(c, tw, exch, t, yv);
+                float2* dst = y + ((long)n * S + s) * DY + t;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+            }
         } else {
             float2* dst = y + s * 64 + t + (long)n * M;          // C[m + n*M], m = s*64 + t + L*i
 #pragma unroll
@@ -176,7 +194,10 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     const int mt = wave & 3, nt0 = (wave >> 2) * NTW;          // m tile, first of the wave's NTW n' tiles
     const long s = blockIdx.x;
     const int n0 = blockIdx.y * 64;
-    float2* exch = lds + g * G::EXCH;
+    // DY = 128: signals are transformed in pairs by 16-lane groups (see the SIMT kernel); COMPACT never applies there
+    constexpr bool PAIR = LOGDY == 7;
+    const int t16 = tid % 16, gpair = (tid / 16) * 2;
+    float2* exch = PAIR ? lds + (tid / 16) * (2 * G::EXCH) : lds + g * G::EXCH;
 
     cpx tw[16];
     const float2* twrow = lds + G::REGION0 + G::REGION1 + t * kTwLdsPitch;
@@ -184,22 +205,29 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
         fill_lds_twiddles<LOGDY>(lds + G::REGION0 + G::REGION1, tid, THREADS);
         __syncthreads();
     } else {
-        load_lane_twiddles<LOGDY>(t, tw);
+        load_lane_twiddles<LOGDY>(PAIR ? t16 : t, tw);
     }
 
     floatx4_1d acc[NTW];
 #pragma unroll
     for (int i = 0; i < NTW; ++i) acc[i] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
 
-    auto issue = [&](cpx (&dst)[16], int k) {
-        const float2* src = x + ((long)k * S + s) * DY + t;
+    // loads of this lane group's channel(s) of the chunk that starts at channel kc
+    auto issue = [&](cpx (&dst)[16], int kc) {
+        if constexpr (PAIR) {
+            const float2* src = x + ((long)(kc + gpair) * S + s) * DY + t16;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = src[L * i];
+            for (int i = 0; i < 8; ++i) { dst[i] = src[16 * i]; dst[8 + i] = src[(long)S * DY + 16 * i]; }
+        } else {
+            const float2* src = x + ((long)(kc + g) * S + s) * DY + t;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[i] = src[L * i];
+        }
     };
     // two chunks of loads in flight per lane group: buffer b receives chunk c + 2 as soon as chunk c has left it
     cpx v0[16], v1[16];
-    if (g < K) issue(v0, g);
-    if (G::DEPTH == 2 && KC + g < K) issue(v1, KC + g);
+    if (g < K) issue(v0, 0);
+    if (G::DEPTH == 2 && KC + g < K) issue(v1, KC);
 
     auto chunk = [&](cpx (&v)[16], int kc) {
         const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
@@ -214,11 +242,19 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
         }
         cpx out[MM];
         if (g < kn) {
-            cpx gg[16];
-            if constexpr (G::COMPACT) fwd_pass1_lds(v, twrow, gg);
-            else fwd_pass1(v, tw, gg);
-            if (kc + G::DEPTH * KC + g < K) issue(v, kc + G::DEPTH * KC + g);    // this group's channel DEPTH chunks ahead
-            group_forward_finish<LOGDY>(gg, exch, t, out);
+            if constexpr (PAIR) {
+                cpx w[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) w[i] = v[i];
+                if (kc + G::DEPTH * KC + g < K) issue(v, kc + G::DEPTH * KC);
+                pair128_forward(w, tw, exch, t16, out);
+            } else {
+                cpx gg[16];
+                if constexpr (G::COMPACT) fwd_pass1_lds(v, twrow, gg);
+                else fwd_pass1(v, tw, gg);
+                if (kc + G::DEPTH * KC + g < K) issue(v, kc + G::DEPTH * KC);    // the chunk DEPTH chunks ahead
+                group_forward_finish<LOGDY>(gg, exch, t, out);
+            }
         }
         __syncthreads();                                       // all exchanges done: sA may overwrite them
         if (g < kn) {
@@ -273,11 +309,18 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     for (int pass = 0; pass < 64 / KC; ++pass) {
         const int n = g + KC * pass;
         cpx yv[16];
-        if constexpr (G::COMPACT) group_backward_lds<LOGDY>(c[pass], twrow, exch, t, yv);
-        else group_backward<LOGDY>(c[pass], tw, exch, t, yv);
-        float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
+        if constexpr (PAIR) {
+            pair128_backward(c[pass], tw, exch, t16, yv);
+            float2* dst = y + ((long)(n0 + gpair + KC * pass) * S + s) * DY + t16;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+            for (int i = 0; i < 8; ++i) { dst[16 * i] = yv[i]; dst[(long)S * DY + 16 * i] = yv[8 + i]; }
+        } else {
+            if constexpr (G::COMPACT) group_backward_lds<LOGDY>(c[pass], twrow, exch, t, yv);
+            else group_backward<LOGDY>(c[pass], tw, exch, t, yv);
+            float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+        }
     }
 }
 
@@ -293,8 +336,46 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x, g = tid / L, t = tid % L;
     const long sig = (long)blockIdx.x * GROUPS + g;
-    float2* exch = lds + g * G::EXCH;
     cpx tw[16];
+    if constexpr (LOGDY == 7) {
+        // signals of 128 samples go in pairs through 16-lane groups (128-byte accesses); lane (g, t) still ends up with /
+        // starts from the modes t + 8 a of signal g. All 16 lanes take part for either signal, so a pair with one
+        // signal beyond nsig loads zeros for it and skips its stores instead of leaving early.
+        const int t16 = tid % 16;
+        const long sigA = (long)blockIdx.x * GROUPS + (tid / 16) * 2;
+        float2* exch = lds + (tid / 16) * (2 * G::EXCH);
+        load_lane_twiddles<LOGDY>(t16, tw);
+        if (sigA >= nsig) return;                    // whole pair out of range (uniform per 16-lane group)
+        const bool hasB = sigA + 1 < nsig;
+        if constexpr (!INVERSE) {
+            const float2* src = in + sigA * DY + t16;
+            cpx v[16], o[MM];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[i] = src[16 * i];
+                v[8 + i] = hasB ? src[DY + 16 * i] : make_float2(0.f, 0.f);
+            }
+            pair128_forward(v, tw, exch, t16, o);
+            if (sig < nsig) {
+                float2* dst = out + sig * 64 + t;
+#pragma unroll
+                for (int a = 0; a < MM; ++a) dst[L * a] = o[a];
+            }
+        } else {
+            cpx c[MM], yv[16];
+#pragma unroll
+            for (int a = 0; a < MM; ++a) c[a] = sig < nsig ? in[sig * 64 + t + L * a] : make_float2(0.f, 0.f);
+            pair128_backward(c, tw, exch, t16, yv);
+            float2* dst = out + sigA * DY + t16;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                dst[16 * i] = yv[i];
+                if (hasB) dst[DY + 16 * i] = yv[8 + i];
+            }
+        }
+        return;
+    } else {
+    float2* exch = lds + g * G::EXCH;
     load_lane_twiddles<LOGDY>(t, tw);
     if (sig >= nsig) return;
     if constexpr (!INVERSE) {
@@ -315,6 +396,7 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
         float2* dst = out + sig * DY + t;
 #pragma unroll
         for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+    }
     }
 }
 
