@@ -4,7 +4,7 @@
 // Replaces fused_fft_cgemm_ifft_{7,8} of the reference
 // (fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused_fft_cgemm_ifft_7.cuh:9-222): same operands
 //   x[K][S][DY]  (signal (k,s) at (k*S+s)*DY),  W[k + n*K],  y[N][S][DY],  M = 64*S,
-// same grid (S, N/64), block 256, and the same "block traverses K" schedule, re-derived for wave64:
+// the same (S, N/64) blocks (as a 1D grid in an XCD-aware order), block 256, and the same "block traverses K" schedule, re-derived for wave64:
 //   * an L = DY/16 lane group owns one signal; a 256-thread block transforms 256/L channels at once
 //     (the reference does 8), so the K loop advances in chunks of 16 (DY=256) or 32 (DY=128) channels;
 //   * the thread that accumulates C[m][n] is the thread that later needs it for the backward
@@ -15,6 +15,25 @@
 #include "kernels.h"
 
 namespace tfno {
+
+// Block -> (signal set s, output tile) for the fused 1D kernels. Consecutive workgroups go to different XCDs (eight L2s),
+// and every output tile of a signal set re-reads the same K input rows: the tiles of one s are therefore given block
+// ids eight apart, which lands them on the same XCD at about the same time, so only the first of them reads x from
+// HBM. Groups of eight signal sets are laid out as [tile][s % 8]; a tail of fewer than eight sets is laid out plainly.
+__device__ __forceinline__ void decode_block_1d(long S, int ntiles, long& s, int& tile)
+{
+    const long id = blockIdx.x, full = (S / 8) * 8;
+    if (id < full * ntiles) {
+        const long grp = id / (8 * ntiles);
+        const int rem = (int)(id % (8 * ntiles));
+        tile = rem / 8;
+        s = grp * 8 + rem % 8;
+    } else {
+        const long rem = id - full * ntiles;
+        s = full + rem / ntiles;
+        tile = (int)(rem % ntiles);
+    }
+}
 
 // FUSE_FWD: the A operand is produced by forward transforms of x (variants B and D); otherwise it is read from
 //           the column-major matrix A[m + k*M] (variant C).
@@ -34,8 +53,10 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 
     const int tid = threadIdx.x;
     const int g = tid / L, t = tid % L;
-    const long s = blockIdx.x;
-    const int n0 = blockIdx.y * 64;
+    long s;
+    int ntile;
+    decode_block_1d(S, N / 64, s, ntile);
+    const int n0 = ntile * 64;
     const long M = 64L * S;
     // signals of 128 samples are transformed in pairs by 16-lane groups (128-byte accesses): lane t16 of pair g/2 holds
     // samples t16 + 16 i of both signals, and ends up with the modes an 8-lane group would give lane (g, t)
@@ -192,8 +213,10 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     const int g = tid / L, t = tid % L;                        // transform role: lane group = channel of the chunk
     const int wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;   // matrix role
     const int mt = wave & 3, nt0 = (wave >> 2) * NTW;          // m tile, first of the wave's NTW n' tiles
-    const long s = blockIdx.x;
-    const int n0 = blockIdx.y * 64;
+    long s;
+    int ntile;
+    decode_block_1d(S, N / 64, s, ntile);
+    const int n0 = ntile * 64;
     // DY = 128: signals are transformed in pairs by 16-lane groups (see the SIMT kernel); COMPACT never applies there
     constexpr bool PAIR = LOGDY == 7;
     const int t16 = tid % 16, gpair = (tid / 16) * 2;
@@ -405,7 +428,8 @@ static hipError_t launch_fused_1d(long S, int N, int K, const float2* x, const f
                                   float2 beta, hipStream_t stream)
 {
     using G = Geo1D<LOGDY>;
-    dim3 grid((unsigned)S, (unsigned)(N / 64), 1), block(256, 1, 1);
+    if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(S * (N / 64)), 1, 1), block(256, 1, 1);
     hipLaunchKernelGGL((fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV>), grid, block, G::LDS_BYTES, stream, (int)S,
                        N, K, x, W, y, alpha, beta);
     return hipGetLastError();
@@ -434,7 +458,8 @@ static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const
                                          G::LDS_BYTES, served);
         e != hipSuccess)
         return e;
-    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS>), dim3((unsigned)S, (unsigned)(N / 64)), dim3(THREADS),
+    if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS>), dim3((unsigned)(S * (N / 64))), dim3(THREADS),
                        G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();
 }
