@@ -49,9 +49,9 @@ def test_config2_sweep_against_oracle(tol):
 
 
 @pytest.mark.parametrize("K", [64, 128])
-@pytest.mark.parametrize("algo", [0, 1, 2])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4])
 def test_config3_large_hidden_against_oracle(K, algo, tol, monkeypatch):
-    """1D bs=64, DY=256, N=128, K in {64, 128}, smooth input: size-chosen kernel, SIMT kernel, matrix-core kernel"""
+    """1D bs=64, DY=256, N=128, K in {64, 128}, smooth input: size-chosen kernel, SIMT kernel, the three matrix-core variants"""
     print("config3", K, algo, flush=True)
     monkeypatch.setenv("TURBOFNO_1D_ALGO", str(algo))
     x, W = workloads.smooth_1d(0x5EED + 3, 64, 256, K, 128)

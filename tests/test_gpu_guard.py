@@ -24,7 +24,7 @@ def intact(buf, what):
     assert bool((lo == CANARY).all()) and bool((hi == CANARY).all()), what + ": guard band overwritten"
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4])
 @pytest.mark.parametrize("bs,DY,K,N", [(3, 256, 72, 128), (5, 128, 40, 64), (1, 256, 8, 64), (7, 128, 136, 128)])
 def test_layer_1d_stays_in_bounds(bs, DY, K, N, algo, monkeypatch):
     print("guard 1d", bs, DY, K, N, algo, flush=True)

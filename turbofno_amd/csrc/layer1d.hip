@@ -177,10 +177,12 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 // sC aliases the W' tile.
 typedef float floatx4_1d __attribute__((ext_vector_type(4)));
 
-template <int LOGDY, int THREADS_> struct GeoMfma1D {
+// NT_ = output channels per block: 64, or 32 to spread a small grid over twice as many CUs (DY = 256, 512 threads).
+template <int LOGDY, int THREADS_, int NT_ = 64> struct GeoMfma1D {
     static constexpr int L = Geo1D<LOGDY>::L, MM = 64 / L;
     static constexpr int THREADS = THREADS_;                  // 512: one block per CU; 256: two (LDS 72 KiB each)
-    static constexpr int NTW = 32 / (THREADS / 64);           // 16x16 tiles per wave: one m tile x NTW n' tiles
+    static constexpr int NT = NT_;
+    static constexpr int NTW = (NT / 2) / (THREADS / 64);     // 16x16 tiles per wave: one m tile x NTW n' tiles
     static constexpr int KC = THREADS / L;                    // channels per chunk = lane groups per block
     // compact: sC shares the exchange regions too and the twiddles move to LDS: 53 KiB and 168 registers, three blocks
     // per CU. Only for DY = 256: at DY = 128 (8 modes per lane) the register limit costs more in spills than it gains.
@@ -189,19 +191,20 @@ template <int LOGDY, int THREADS_> struct GeoMfma1D {
     static constexpr int EXCH = L * 17;
     static constexpr int REGION0 = KC * EXCH > KC * PA ? KC * EXCH : KC * PA;              // exchange | sA
     static constexpr int WTILE = (KC / 4) * kWGroup / 2;                                   // W' tile in complex units
-    static constexpr int REGION1 = COMPACT ? WTILE : (WTILE > 64 * PC ? WTILE : 64 * PC);  // W' | sC   (complex)
-    static_assert(!COMPACT || 64 * PC <= REGION0, "sC must fit the exchange regions");
+    static constexpr int REGION1 = COMPACT ? WTILE : (WTILE > NT * PC ? WTILE : NT * PC);  // W' | sC   (complex)
+    static_assert(!COMPACT || NT * PC <= REGION0, "sC must fit the exchange regions");
+    static_assert(NT == 64 || (NT == 32 && THREADS_ == 512 && LOGDY == 8), "32-channel tiles: DY = 256, 512 threads");
     static constexpr int TWTAB = COMPACT ? kTwLdsSize : 0;    // compact: twiddles in LDS instead of 30 registers
     static constexpr int DEPTH = COMPACT ? 1 : 2;             // chunks of loads in flight per lane group
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1 + TWTAB);
 };
 
-template <int LOGDY, int THREADS>
+template <int LOGDY, int THREADS, int NT>
 __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                       const float2* __restrict__ W, float2* __restrict__ y,
                                                                       float2 alpha)
 {
-    using G = GeoMfma1D<LOGDY, THREADS>;
+    using G = GeoMfma1D<LOGDY, THREADS, NT>;
     constexpr int NTW = G::NTW;
     constexpr int DY = 1 << LOGDY, L = G::L, MM = G::MM, KC = G::KC, PA = G::PA, PC = G::PC;
     extern __shared__ float2 lds[];
@@ -215,8 +218,8 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     const int mt = wave & 3, nt0 = (wave >> 2) * NTW;          // m tile, first of the wave's NTW n' tiles
     long s;
     int ntile;
-    decode_block_1d(S, N / 64, s, ntile);
-    const int n0 = ntile * 64;
+    decode_block_1d(S, N / NT, s, ntile);
+    const int n0 = ntile * NT;
     // DY = 128: signals are transformed in pairs by 16-lane groups (see the SIMT kernel); COMPACT never applies there
     constexpr bool PAIR = LOGDY == 7;
     const int t16 = tid % 16, gpair = (tid / 16) * 2;
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     auto chunk = [&](cpx (&v)[16], int kc) {
         const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
         // W chunk: lanes run along k, the contiguous direction of W[k + n*K]
-        constexpr int WPT = KC * 64 / G::THREADS;
+        constexpr int WPT = KC * NT / G::THREADS;
         float2 wv[WPT];
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
@@ -322,14 +325,14 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     __syncthreads();
     // every pass takes its modes before the first backward transform: in the compact layout the exchange regions
     // overlay sC
-    cpx c[64 / KC][MM];
+    cpx c[NT / KC][MM];
 #pragma unroll
-    for (int pass = 0; pass < 64 / KC; ++pass)
+    for (int pass = 0; pass < NT / KC; ++pass)
 #pragma unroll
         for (int a = 0; a < MM; ++a) c[pass][a] = sC[(g + KC * pass) * PC + t + L * a];
     if constexpr (G::COMPACT) __syncthreads();
 #pragma unroll
-    for (int pass = 0; pass < 64 / KC; ++pass) {
+    for (int pass = 0; pass < NT / KC; ++pass) {
         const int n = g + KC * pass;
         cpx yv[16];
         if constexpr (PAIR) {
@@ -448,18 +451,18 @@ static hipError_t dispatch_fused_1d(int logDY, long S, int N, int K, const float
     }
 }
 
-template <int LOGDY, int THREADS>
+template <int LOGDY, int THREADS, int NT = 64>
 static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
                                     hipStream_t stream)
 {
-    using G = GeoMfma1D<LOGDY, THREADS>;
+    using G = GeoMfma1D<LOGDY, THREADS, NT>;
     static std::atomic<unsigned long long> served;
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY, THREADS>),
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT>),
                                          G::LDS_BYTES, served);
         e != hipSuccess)
         return e;
-    if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS>), dim3((unsigned)(S * (N / 64))), dim3(THREADS),
+    if (S * (N / NT) > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT>), dim3((unsigned)(S * (N / NT))), dim3(THREADS),
                        G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();
 }
@@ -474,11 +477,14 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
     //    its vector instructions there, more than half of which are the contraction;
     //  * otherwise the SIMT kernel (three blocks per CU, no idle lanes in short chunks).
-    int pick = algo;
+    int pick = algo == 4 ? 2 : algo;             // 4 = matrix cores, 512 threads, 32-channel tiles (DY = 256 only)
     if (pick == 0) {
         const bool fills = (logDY == 8 && K >= 32) || (logDY == 7 && K >= 64);
         pick = (fills && S * (N / 64) <= cu_count()) ? 2 : (K >= 64 ? 3 : 1);
     }
+    // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
+    if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
+        return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream);
     if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream);
     if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream);
     if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream);
