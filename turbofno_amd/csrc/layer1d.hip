@@ -471,19 +471,16 @@ static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
-    // by size (measured crossovers on MI355X):
-    //  * while every block has a CU to itself and the 512-thread kernel needs fewer chunks: matrix cores, 8 waves per
-    //    block (the shortest chain of latencies);
+    // by size (measured on MI355X):
+    //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
+    //    every K, even K = 8 where most of a chunk is padding;
     //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
     //    its vector instructions there, more than half of which are the contraction;
     //  * otherwise the SIMT kernel (three blocks per CU, no idle lanes in short chunks).
     int pick = algo == 4 ? 2 : algo;             // 4 = matrix cores, 512 threads, 32-channel tiles (DY = 256 only)
     if (pick == 0) {
-        // "fills": the 512-thread kernel needs fewer chunks than the SIMT kernel (chunks of 32 vs 16 channels at
-        // DY = 256, 64 vs 32 at DY = 128)
-        const int kc_simt = logDY == 8 ? 16 : 32;
-        const bool fills = (logDY == 7 || logDY == 8) && (K + 2 * kc_simt - 1) / (2 * kc_simt) < (K + kc_simt - 1) / kc_simt;
-        pick = (fills && S * (N / 64) <= cu_count()) ? 2 : (K >= 64 ? 3 : 1);
+        const bool built = logDY == 7 || logDY == 8;
+        pick = (built && S * (N / 64) <= cu_count()) ? 2 : (K >= 64 ? 3 : 1);
     }
     // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
