@@ -474,13 +474,13 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     // by size (measured on MI355X):
     //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
     //    every K, even K = 8 where most of a chunk is padding;
-    //  * larger grids with K >= 64: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
-    //    its vector instructions there, more than half of which are the contraction;
-    //  * otherwise the SIMT kernel (three blocks per CU, no idle lanes in short chunks).
+    //  * larger grids with K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
+    //    its vector instructions there, up to half of which are the contraction;
+    //  * larger grids with K < 32: the SIMT kernel (three blocks per CU, no idle lanes in short chunks; a tie at K = 16).
     int pick = algo == 4 ? 2 : algo;             // 4 = matrix cores, 512 threads, 32-channel tiles (DY = 256 only)
     if (pick == 0) {
         const bool built = logDY == 7 || logDY == 8;
-        pick = (built && S * (N / 64) <= cu_count()) ? 2 : (K >= 64 ? 3 : 1);
+        pick = (built && S * (N / 64) <= cu_count()) ? 2 : (K >= 32 ? 3 : 1);
     }
     // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
