@@ -39,7 +39,7 @@ def test_shipped_configs_parse(config_check):
 
 
 @pytest.mark.gpu
-def test_driver_result_lines():
+def test_driver_result_lines(tmp_path):
     exe1, exe2 = os.path.join(ROOT, "bin", "TurboFNO_1D_D"), os.path.join(ROOT, "bin", "TurboFNO_2D_D")
     assert os.path.exists(exe1) and os.path.exists(exe2), "build the drivers with make -C turbofno_amd/host"
     out = subprocess.run([exe1, "4", "1", "128", "64", "16"], check=True, capture_output=True, text=True, timeout=100).stdout
@@ -49,8 +49,7 @@ def test_driver_result_lines():
     print(out, flush=True)
     assert re.fullmatch(r"2D_D, bs=1   , DX=256 , DY=256 , N=64  , K=16  , TIME=\s*\d+\.\d{3}ms\n", out), out
     # config-file mode: a tiny grid, loop order bs -> DX -> DY -> N -> K
-    cfg = os.path.join(ROOT, "gpurun_out", "tiny_2d.txt")
-    os.makedirs(os.path.dirname(cfg), exist_ok=True)
+    cfg = str(tmp_path / "tiny_2d.txt")
     with open(cfg, "w") as f:
         f.write("bs_list = 1\nDX_list = 128 256\nDY_list = 128\nN_list = 64\nK_list = 8 16")
     lines = subprocess.run([exe2, cfg], check=True, capture_output=True, text=True, timeout=100).stdout.splitlines()
