@@ -256,7 +256,8 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 //   C[n][m] = alpha * sum_k W[k + n*K] * A[k][m],   A: [K][Mtot], C: [N][Mtot]  (m contiguous)
 // Same contraction as the reference's cgemm / the GEMM phase of its fused kernel
 // (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4-205, operand layout lda=M, ldb=K, ldc=M),
-// expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition) on
+// expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition; for 16 < K <= 64 the
+// three-product form of cgemm_modes3m_kernel below is used instead) on
 // v_mfma_f32_16x16x4_f32: rows = (n, re/im), cols = 16 consecutive m, contraction = 4 channels x re|im.
 // A block is 16 waves; wave w owns the 16-m strip w and the whole 64-channel n tile (8 accumulators of
 // 16x16), so every element of A is loaded exactly once: the strip of a 64-channel chunk sits in 16 float2
@@ -360,6 +361,75 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     }
 }
 
+// The same contraction for K <= 64 (one chunk) with three real products per complex one instead of four:
+//   P1 = c (a + b),  P2 = (d - c) a,  P3 = (c + d) b   =>   re = P1 - P3,  im = P1 + P2      (W' = c + i d, A = a + i b)
+// i.e. three matrix instructions per 16 n x 16 m x 4 k instead of four: 25 % less matrix work, and the matrix work is
+// the part of this kernel that nothing overlaps with. Rows of a tile are 16 output channels n (not 8 x re|im); per n
+// tile a wave keeps only the three accumulators P1, P2, P3 and stores the tile when it is complete.
+// W'' tile in LDS: float4 {c, d - c, c + d, unused} at float index (k * kW3Row + n * 4): an operand fetch of 16 n for
+// one k is 256 contiguous bytes; rows of different k are padded by four floats so that the build (lanes along k) does
+// not put a whole wavefront on one bank.
+constexpr int kW3Row = 64 * 4 + 4;
+
+template <int NG>
+__global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float2* __restrict__ A,
+                                                                     const float2* __restrict__ W, float2* __restrict__ C,
+                                                                     long Mtot, int N, int K, float2 alpha, float2 beta)
+{
+    extern __shared__ float sW[];                     // GEMM_KC * kW3Row floats
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.y * 64;
+    const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
+    const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
+    const bool active = (long)blockIdx.x * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
+    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
+    const bool has_beta = beta.x != 0.f || beta.y != 0.f;
+
+    // the wave's whole A strip: lane (kq, col) holds channels 4 g + kq, g < NG
+    float2 bv[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+        bv[g] = (active && 4 * g < K) ? (blk + (long)(4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+    // W'' tile: lanes run along k, the contiguous direction of W[k + n*K]
+    constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
+    float2 wv[WPT];
+#pragma unroll
+    for (int u = 0; u < WPT; ++u) {
+        const int idx = tid + u * GEMM_THREADS;
+        const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+        wv[u] = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < WPT; ++u) {
+        const int idx = tid + u * GEMM_THREADS;
+        const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+        const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+        *reinterpret_cast<float4*>(&sW[k * kW3Row + n * 4]) = make_float4(c, d - c, c + d, 0.f);
+    }
+    __syncthreads();
+    if (!active) return;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        floatx4 p1 = { 0.f, 0.f, 0.f, 0.f }, p2 = p1, p3 = p1;
+        const float* wrow = &sW[kq * kW3Row + (t * 16 + col) * 4];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            const float4 w = *reinterpret_cast<const float4*>(wrow + g * 4 * kW3Row);
+            p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bv[g].x + bv[g].y, p1, 0, 0, 0);
+            p2 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bv[g].x, p2, 0, 0, 0);
+            p3 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bv[g].y, p3, 0, 0, 0);
+        }
+        // D[row = 4 kq + v][col]: output channel n0 + 16 t + 4 kq + v, column m = wave * 16 + col
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float2* p = cblk + (long)(n0 + 16 * t + 4 * kq + v) * Mtot + (wave * 16 + col);
+            float2 r = make_float2(p1[v] - p3[v], p1[v] + p2[v]);
+            if (has_beta) r = cadd(r, cmul(*p, beta));
+            *p = r;
+        }
+    }
+}
+
 int cu_count()
 {
     static std::atomic<int> cached[64];
@@ -427,6 +497,23 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         hipLaunchKernelGGL(cgemm_modes_kernel<NG>, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
         return hipGetLastError();
     };
+    // one chunk of more than 16 channels: three real products per complex one (25 % less matrix work); K <= 16 is
+    // bound by the tile build and the stores, K > 64 needs the accumulators of all tiles across chunks
+    if (K > 16 && K <= GEMM_KC) {
+        constexpr size_t bytes3 = sizeof(float) * GEMM_KC * kW3Row;
+        auto launch3 = [&](auto ng_const) -> hipError_t {
+            constexpr int NG = decltype(ng_const)::value;
+            static std::atomic<unsigned long long> served3;
+            if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_kernel<NG>), bytes3, served3);
+                e != hipSuccess)
+                return e;
+            hipLaunchKernelGGL(cgemm_modes3m_kernel<NG>, grid, dim3(GEMM_THREADS), bytes3, stream, A, W, C, Mtot, N, K, alpha, beta);
+            return hipGetLastError();
+        };
+        if (K <= 32) return launch3(std::integral_constant<int, 8>{});
+        if (K <= 48) return launch3(std::integral_constant<int, 12>{});
+        return launch3(std::integral_constant<int, 16>{});
+    }
     if (K <= 16) return launch(std::integral_constant<int, 4>{});
     if (K <= 32) return launch(std::integral_constant<int, 8>{});
     if (K <= 48) return launch(std::integral_constant<int, 12>{});
