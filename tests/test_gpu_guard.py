@@ -52,7 +52,7 @@ def test_layer_2d_stays_in_bounds(bs, DX, DY, K, N, algo):
     assert not bool((y == CANARY).any())
 
 
-@pytest.mark.parametrize("M,N,K", [(64, 64, 8), (192, 128, 72), (4160, 64, 16), (1024, 64, 48)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 8), (192, 128, 72), (4160, 64, 16), (1024, 64, 48), (320, 64, 128)])
 def test_cgemm_stays_in_bounds(M, N, K):
     print("guard cgemm", M, N, K, flush=True)
     rng = np.random.default_rng(M + K)

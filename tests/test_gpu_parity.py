@@ -90,7 +90,11 @@ def test_stride_stages(DX, DY, nsig, tol):
     (1, 256, 256, 16, 64, 1),
     (1, 256, 256, 16, 64, 2),
     (2, 256, 256, 8, 128, 2),
-    (1, 256, 256, 72, 64, 2),        # K crosses the 64-channel W chunk of the matrix-core GEMM
+    (1, 256, 256, 72, 64, 2),        # K above 64: GEMM in chunks of 32 channels (32 + 32 + 8)
+    (1, 128, 128, 128, 64, 2),       # four full chunks
+    (1, 128, 128, 104, 128, 2),      # 32 + 32 + 32 + 8, two N tiles
+    (1, 128, 128, 40, 64, 2),        # one chunk, 12 channel groups (last one half empty)
+    (1, 128, 128, 64, 64, 2),        # one full chunk
     (1, 128, 128, 16, 64, 2),        # whole-image kernels for the other three built shapes
     (3, 128, 256, 8, 64, 2),
     (2, 256, 128, 24, 128, 2),
@@ -138,7 +142,7 @@ def test_error_codes():
 
 
 @pytest.mark.parametrize("S,DY,K,N", [(4, 128, 8, 64), (8, 256, 24, 128), (1, 128, 16, 64), (5, 256, 8, 64),
-                                      (3, 512, 16, 64), (2, 1024, 8, 64)])
+                                      (3, 512, 16, 64), (2, 1024, 8, 64), (5, 128, 64, 64), (3, 128, 104, 128)])
 def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     """stages of variants A, B, C: contiguous transforms, cgemm with beta, the two half-fused kernels"""
     print("case variant stages", S, DY, K, N, flush=True)

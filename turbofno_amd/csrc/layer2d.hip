@@ -361,17 +361,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
     }
 }
 
-// The same contraction for K <= 64 (one chunk) with three real products per complex one instead of four:
+// The same contraction with three real products per complex one instead of four:
 //   P1 = c (a + b),  P2 = (d - c) a,  P3 = (c + d) b   =>   re = P1 - P3,  im = P1 + P2      (W' = c + i d, A = a + i b)
 // i.e. three matrix instructions per 16 n x 16 m x 4 k instead of four: 25 % less matrix work, and the matrix work is
-// the part of this kernel that nothing overlaps with. Rows of a tile are 16 output channels n (not 8 x re|im); per n
-// tile a wave keeps only the three accumulators P1, P2, P3 and stores the tile when it is complete.
+// the part of this kernel that nothing overlaps with. Rows of a tile are 16 output channels n (not 8 x re|im); a wave
+// keeps the accumulators P1, P2, P3 of its four n tiles and stores a tile when its last chunk is done.
 // W'' tile in LDS: float4 {c, d - c, c + d, unused} at float index (k * kW3Row + n * 4): an operand fetch of 16 n for
 // one k is 256 contiguous bytes; rows of different k are padded by four floats so that the build (lanes along k) does
 // not put a whole wavefront on one bank.
 constexpr int kW3Row = 64 * 4 + 4;
 
-template <int NG>
+template <int NG, bool MULTI>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float2* __restrict__ A,
                                                                      const float2* __restrict__ W, float2* __restrict__ C,
                                                                      long Mtot, int N, int K, float2 alpha, float2 beta)
@@ -385,47 +385,69 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
     float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
     const bool has_beta = beta.x != 0.f || beta.y != 0.f;
 
-    // the wave's whole A strip: lane (kq, col) holds channels 4 g + kq, g < NG
-    float2 bv[NG];
+    floatx4 p1[4], p2[4], p3[4];
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
-        bv[g] = (active && 4 * g < K) ? (blk + (long)(4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
-    // W'' tile: lanes run along k, the contiguous direction of W[k + n*K]
-    constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
-    float2 wv[WPT];
+    for (int t = 0; t < 4; ++t) p1[t] = p2[t] = p3[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
+
+    // one chunk of up to 64 channels, or (MULTI) chunks of 4 NG = 32 channels with the accumulators kept across them
+    constexpr int KCH = MULTI ? 4 * NG : GEMM_KC;
+    for (int kc = 0; kc < (MULTI ? K : 1); kc += KCH) {
+        const int kn = (K - kc) < KCH ? (K - kc) : KCH;           // multiple of 8 (caller contract)
+        const bool last = !MULTI || kc + KCH >= K;
+        // the wave's whole A strip of this chunk: lane (kq, col) holds channels kc + 4 g + kq, g < NG
+        // (with one chunk the loads are issued before the tile build and overlap it; with several, the accumulators
+        // of all tiles stay live and the strip is loaded after the build to stay inside 128 registers)
+        float2 bv[NG];
+        if constexpr (!MULTI) {
 #pragma unroll
-    for (int u = 0; u < WPT; ++u) {
-        const int idx = tid + u * GEMM_THREADS;
-        const int k = idx % GEMM_KC, n = idx / GEMM_KC;
-        wv[u] = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
-    }
-#pragma unroll
-    for (int u = 0; u < WPT; ++u) {
-        const int idx = tid + u * GEMM_THREADS;
-        const int k = idx % GEMM_KC, n = idx / GEMM_KC;
-        const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
-        *reinterpret_cast<float4*>(&sW[k * kW3Row + n * 4]) = make_float4(c, d - c, c + d, 0.f);
-    }
-    __syncthreads();
-    if (!active) return;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        floatx4 p1 = { 0.f, 0.f, 0.f, 0.f }, p2 = p1, p3 = p1;
-        const float* wrow = &sW[kq * kW3Row + (t * 16 + col) * 4];
-#pragma unroll
-        for (int g = 0; g < NG; ++g) {
-            const float4 w = *reinterpret_cast<const float4*>(wrow + g * 4 * kW3Row);
-            p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bv[g].x + bv[g].y, p1, 0, 0, 0);
-            p2 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bv[g].x, p2, 0, 0, 0);
-            p3 = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bv[g].y, p3, 0, 0, 0);
+            for (int g = 0; g < NG; ++g)
+                bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         }
-        // D[row = 4 kq + v][col]: output channel n0 + 16 t + 4 kq + v, column m = wave * 16 + col
+        __syncthreads();                              // the previous chunk's tile is no longer read
+        // W'' tile: lanes run along k, the contiguous direction of W[k + n*K]
+        constexpr int WPT = KCH * 64 / GEMM_THREADS;
+        float2 wv[WPT];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            float2* p = cblk + (long)(n0 + 16 * t + 4 * kq + v) * Mtot + (wave * 16 + col);
-            float2 r = make_float2(p1[v] - p3[v], p1[v] + p2[v]);
-            if (has_beta) r = cadd(r, cmul(*p, beta));
-            *p = r;
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
+            const int k = idx % KCH, n = idx / KCH;
+            wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
+            const int k = idx % KCH, n = idx / KCH;
+            const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+            *reinterpret_cast<float4*>(&sW[k * kW3Row + n * 4]) = make_float4(c, d - c, c + d, 0.f);
+        }
+        if constexpr (MULTI) {
+#pragma unroll
+            for (int g = 0; g < NG; ++g)
+                bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+        }
+        __syncthreads();
+        if (!active) continue;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if constexpr (!MULTI) p1[t] = p2[t] = p3[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
+            const float* wrow = &sW[kq * kW3Row + (t * 16 + col) * 4];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                const float4 w = *reinterpret_cast<const float4*>(wrow + g * 4 * kW3Row);
+                p1[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bv[g].x + bv[g].y, p1[t], 0, 0, 0);
+                p2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bv[g].x, p2[t], 0, 0, 0);
+                p3[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bv[g].y, p3[t], 0, 0, 0);
+            }
+            if (last) {
+                // D[row = 4 kq + v][col]: output channel n0 + 16 t + 4 kq + v, column m = wave * 16 + col
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float2* p = cblk + (long)(n0 + 16 * t + 4 * kq + v) * Mtot + (wave * 16 + col);
+                    float2 r = make_float2(p1[t][v] - p3[t][v], p1[t][v] + p2[t][v]);
+                    if (has_beta) r = cadd(r, cmul(*p, beta));      // C = alpha A W + beta C (variants A, B)
+                    *p = r;
+                }
+            }
         }
     }
 }
@@ -497,27 +519,27 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         hipLaunchKernelGGL(cgemm_modes_kernel<NG>, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
         return hipGetLastError();
     };
-    // one chunk of more than 16 channels: three real products per complex one (25 % less matrix work); K <= 16 is
-    // bound by the tile build and the stores, K > 64 needs the accumulators of all tiles across chunks
-    if (K > 16 && K <= GEMM_KC) {
+    // more than 16 channels: three real products per complex one (25 % less matrix work); K <= 16 is bound by the
+    // tile build and the stores, where the four-product kernel is slightly faster
+    if (K > 16) {
         constexpr size_t bytes3 = sizeof(float) * GEMM_KC * kW3Row;
-        auto launch3 = [&](auto ng_const) -> hipError_t {
+        auto launch3 = [&](auto ng_const, auto multi_const) -> hipError_t {
             constexpr int NG = decltype(ng_const)::value;
+            constexpr bool MULTI = decltype(multi_const)::value;
             static std::atomic<unsigned long long> served3;
-            if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_kernel<NG>), bytes3, served3);
+            if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_kernel<NG, MULTI>), bytes3, served3);
                 e != hipSuccess)
                 return e;
-            hipLaunchKernelGGL(cgemm_modes3m_kernel<NG>, grid, dim3(GEMM_THREADS), bytes3, stream, A, W, C, Mtot, N, K, alpha, beta);
+            hipLaunchKernelGGL((cgemm_modes3m_kernel<NG, MULTI>), grid, dim3(GEMM_THREADS), bytes3, stream, A, W, C, Mtot, N, K,
+                               alpha, beta);
             return hipGetLastError();
         };
-        if (K <= 32) return launch3(std::integral_constant<int, 8>{});
-        if (K <= 48) return launch3(std::integral_constant<int, 12>{});
-        return launch3(std::integral_constant<int, 16>{});
+        if (K <= 32) return launch3(std::integral_constant<int, 8>{}, std::false_type{});
+        if (K <= 48) return launch3(std::integral_constant<int, 12>{}, std::false_type{});
+        if (K <= GEMM_KC) return launch3(std::integral_constant<int, 16>{}, std::false_type{});
+        return launch3(std::integral_constant<int, 8>{}, std::true_type{});
     }
-    if (K <= 16) return launch(std::integral_constant<int, 4>{});
-    if (K <= 32) return launch(std::integral_constant<int, 8>{});
-    if (K <= 48) return launch(std::integral_constant<int, 12>{});
-    return launch(std::integral_constant<int, 16>{});
+    return launch(std::integral_constant<int, 4>{});
 }
 
 }  // namespace tfno
