@@ -46,7 +46,7 @@ def test_layer_1d(bs, DY, K, N, alpha, tol):
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d")
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5])
 @pytest.mark.parametrize("bs,DY,K,N,alpha", [
     (2, 256, 32, 64, 1.0),           # exactly one chunk of the matrix-core kernel
     (3, 256, 72, 128, 1 - 1j),       # chunks 32 + 32 + 8, two N tiles
@@ -63,6 +63,21 @@ def test_layer_1d_both_contractions(bs, DY, K, N, alpha, algo, tol, monkeypatch)
     y = tf.layer_1d(dev(x), dev(W), alpha=alpha)
     torch.cuda.synchronize()
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d algo %d" % algo)
+
+
+@pytest.mark.parametrize("bs,DY,K,N", [
+    (1030, 128, 16, 64),             # DY=128: from two items per CU on for K <= 16
+    (600, 128, 40, 128),             # DY=128, 1200 items, K = 5 rounds of 8 channels
+    (2100, 256, 8, 64),              # DY=256: from eight items per CU on
+    (1040, 256, 72, 128),            # DY=256, 2080 items, two N tiles, K = 18 rounds of 4 channels
+])
+def test_layer_1d_large_grids(bs, DY, K, N, tol):
+    """grids large enough for the size rule to pick the one-wavefront-per-item kernel (on a 256-CU device)"""
+    print("case layer_1d large grid", bs, DY, K, N, flush=True)
+    x, W = workloads.uniform_1d(3 + bs + DY + K, bs, DY, K, N)
+    y = tf.layer_1d(dev(x), dev(W), alpha=1 - 1j)
+    torch.cuda.synchronize()
+    check(y, oracle.layer_1d(x, W, 1 - 1j), tol, "layer_1d large grid")
 
 
 @pytest.mark.parametrize("DX,DY,nsig", [(128, 128, 3), (256, 128, 2), (128, 256, 2), (256, 256, 2),

@@ -70,12 +70,13 @@ const char* turbofno_last_error_string(void) { return g_err; }
 
 // The fused 1D entry point keeps the reference's kernel signature, which has no room for an algorithm selector:
 // TURBOFNO_1D_ALGO in the environment (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with 512- / 256-thread
-// blocks, 4 matrix cores with 512 threads and 32-channel output tiles) overrides the choice.
+// blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one wavefront per signal
+// set and output tile) overrides the choice.
 static int algo_1d()
 {
     const char* e = getenv("TURBOFNO_1D_ALGO");
     const int a = e ? atoi(e) : 0;
-    return (a >= 1 && a <= 4) ? a : 0;
+    return (a >= 1 && a <= 5) ? a : 0;
 }
 
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,

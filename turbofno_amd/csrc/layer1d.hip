@@ -142,12 +142,12 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
                 pair128_backward(c, tw, exch, t16, yv);
                 float2* dst = y + ((long)(n0 + gpair + GROUPS * j) * S + s) * DY + t16;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) { dst[16 * i] = yv[i]; dst[(long)S * DY + 16 * i] = yv[8 + i]; }
+                for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
             } else {
                 group_backward<LOGDY>(c, tw, exch, t, yv);
                 float2* dst = y + ((long)n * S + s) * DY + t;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+                for (int i = 0; i < 16; ++i) store_streaming(dst + L * i, yv[i]);
             }
         } else {
             float2* dst = y + s * 64 + t + (long)n * M;          // C[m + n*M], m = s*64 + t + L*i
@@ -339,13 +339,182 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
             pair128_backward(c[pass], tw, exch, t16, yv);
             float2* dst = y + ((long)(n0 + gpair + KC * pass) * S + s) * DY + t16;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { dst[16 * i] = yv[i]; dst[(long)S * DY + 16 * i] = yv[8 + i]; }
+            for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
         } else {
             if constexpr (G::COMPACT) group_backward_lds<LOGDY>(c[pass], twrow, exch, t, yv);
             else group_backward<LOGDY>(c[pass], tw, exch, t, yv);
             float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+            for (int i = 0; i < 16; ++i) store_streaming(dst + L * i, yv[i]);
+        }
+    }
+}
+
+// Fused 1D layer for large grids, DY = 128 / 256: ONE WAVEFRONT per (signal set, 64 output channels), no block barrier
+// and no staging of operands through LDS. The register layouts of the transforms and of v_mfma_f32_16x16x4_f32 coincide:
+//   * DY = 256: the four 16-lane groups of a wave transform four channels k = kc + g at a time and lane (g, t) ends up
+//     with modes t + 16 a, a < 4, of channel g: exactly the B operand (k = lane / 16, column = lane % 16) of the four
+//     m tiles a;
+//   * the A operand row n' = 16 nt + t, k = g is one element of W (times alpha, as (re, -im) or (im, re)), read
+//     straight from global memory (W is a few KiB and stays in the vector cache);
+//   * the accumulators D[row = 4 g + v][column = t] of tile (nt, a) hold, for j = 0, 1, the complex value
+//     (v = 2 j, 2 j + 1) of output channel n = 8 nt + 2 g + j at mode t + 16 a: the input layout of the zero-padded
+//     backward transform of channel n by lane group g;
+//   * DY = 128: a lane group transforms two channels kc + 2 g + h at a time (lane t = r + 8 h finishes channel h with
+//     modes r + 8 c, c < 8); one exchange between lanes t and t ^ 8 (a row rotation, no LDS) turns that into modes
+//     t + 16 a of each of the two channels, i.e. two B operands, and the same exchange leads from the accumulators to
+//     the paired backward transform of output channels 8 nt + 2 g and 8 nt + 2 g + 1.
+// 32 accumulator tiles (128 registers) per wave, two waves per SIMD; the only LDS traffic left is the exchange inside
+// the transforms. The loads of the next channels are issued as soon as the first pass has consumed the current ones
+// and travel under the exchange, the second pass and the matrix instructions (64 per four channels).
+TFNO_DEV float rotate8(float v)        // value of lane t ^ 8 of the same 16-lane row
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+}
+TFNO_DEV cpx rotate8(cpx v) { return make_float2(rotate8(v.x), rotate8(v.y)); }
+
+template <int LOGDY>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fused_fft_mfma_ifft_wave_kernel(
+    int S, int N, int K, const float2* __restrict__ x, const float2* __restrict__ W, float2* __restrict__ y, float2 alpha)
+{
+    constexpr int DY = 1 << LOGDY, EXCH = 16 * 17;
+    constexpr bool PAIR = LOGDY == 7;
+    constexpr int CH = PAIR ? 8 : 4;                              // channels per round
+    __shared__ float2 lds[8 * EXCH + kTwLdsSize];
+    const int lane = threadIdx.x, g = lane >> 4, t = lane & 15;
+    float2* exch = lds + g * EXCH;
+    float2* exch1 = exch + 4 * EXCH;                              // second region: two backward transforms in flight
+    float2* twtab = lds + 8 * EXCH;
+    fill_lds_twiddles<LOGDY>(twtab, lane, 64);
+    const float2* twrow = twtab + t * kTwLdsPitch;
+    __syncthreads();
+    long s;
+    int ntile;
+    decode_block_1d(S, N / 64, s, ntile);
+    const int n0 = ntile * 64;
+    const bool upper = t >> 3, odd = t & 1;
+
+    floatx4_1d acc[8][4];
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) acc[nt][a] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
+
+    // lane (g, t): samples t + 16 i of channel kc + g (DY = 256) or of channels kc + 2 g, kc + 2 g + 1 (DY = 128)
+    const float2* src = x + ((long)(PAIR ? 2 * g : g) * S + s) * DY + t;
+    const float2* wsrc = W + (PAIR ? 2 * g : g) + (long)(n0 + (t >> 1)) * K;   // W[k][n = n0 + 8 nt + t / 2]
+    auto issue = [&](cpx (&dst)[16]) {
+        if constexpr (PAIR) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { dst[i] = src[16 * i]; dst[8 + i] = src[(long)S * DY + 16 * i]; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[i] = src[16 * i];
+        }
+    };
+    // one complex product row: acc += W'(row n', k) x B(k, column), W' = alpha W as (re, -im) / (im, re) by row parity
+    auto contract = [&](floatx4_1d (&d)[4], float2 wk, const cpx (&b)[4]) {
+        const float2 w = make_float2(wk.x * alpha.x - wk.y * alpha.y, wk.x * alpha.y + wk.y * alpha.x);
+        const float ax = odd ? w.y : w.x, ay = odd ? w.x : -w.y;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            d[a] = __builtin_amdgcn_mfma_f32_16x16x4f32(ax, b[a].x, d[a], 0, 0, 0);
+            d[a] = __builtin_amdgcn_mfma_f32_16x16x4f32(ay, b[a].y, d[a], 0, 0, 0);
+        }
+    };
+    cpx v[16];
+    issue(v);
+    for (int kc = 0; kc < K; kc += CH) {                          // K is a multiple of 8 (caller contract)
+        float2 wv[8], wv1[8];
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) {
+            wv[nt] = wsrc[kc + (long)(8 * nt) * K];
+            if constexpr (PAIR) wv1[nt] = wsrc[kc + 1 + (long)(8 * nt) * K];
+        }
+        if constexpr (!PAIR) {
+            cpx gg[16], out[4];
+            fwd_pass1_lds(v, twrow, gg);
+            if (kc + CH < K) { src += (long)CH * S * DY; issue(v); }
+            group_forward_finish<8>(gg, exch, t, out);
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) contract(acc[nt], wv[nt], out);
+        } else {
+            cpx gg[16], out[8], b8[8];
+            {
+                cpx a8[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { a8[i] = v[i]; b8[i] = v[8 + i]; }
+                fft8<-1>(a8);
+                fft8<-1>(b8);
+#pragma unroll
+                for (int r = 0; r < 8; ++r) gg[r] = a8[r];
+            }
+            if (kc + CH < K) { src += (long)CH * S * DY; issue(v); }
+            gg[8] = b8[0];
+#pragma unroll
+            for (int r = 1; r < 8; ++r) {
+                const cpx w = twrow[r];
+                gg[r] = cmul(gg[r], w);
+                gg[8 + r] = cmul(b8[r], w);
+            }
+            rows128_forward_finish(gg, exch, t, out);             // out[c] = mode (t & 7) + 8 c of channel t >> 3
+            // lanes t < 8 keep the even c of their channel and take the even c of the other one; lanes t >= 8 the odd c
+            cpx b0[4], b1[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const cpx got = rotate8(upper ? out[2 * a] : out[2 * a + 1]);
+                b0[a] = upper ? got : out[2 * a];                 // channel kc + 2 g,     mode t + 16 a
+                b1[a] = upper ? out[2 * a + 1] : got;             // channel kc + 2 g + 1, mode t + 16 a
+            }
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                contract(acc[nt], wv[nt], b0);
+                contract(acc[nt], wv1[nt], b1);
+            }
+        }
+    }
+    // backward: the two output channels (j = 0, 1) a lane group owns per n tile are transformed together
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) {
+        cpx c0[4], c1[4], y0[16], y1[16];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            c0[a] = make_float2(acc[nt][a][0], acc[nt][a][1]);   // channel 8 nt + 2 g,     mode t + 16 a
+            c1[a] = make_float2(acc[nt][a][2], acc[nt][a][3]);   // channel 8 nt + 2 g + 1, mode t + 16 a
+        }
+        float2* dst = y + ((long)(n0 + 8 * nt + 2 * g) * S + s) * DY + t;
+        if constexpr (!PAIR) {
+            // each through its own exchange region, so that the LDS round trips of one overlap the arithmetic of the other
+            cpx h0[16], h1[16], e0[16], e1[16];
+            dft16_pad4<+1>(c0, h0);
+            dft16_pad4<+1>(c1, h1);
+            wave_lds_fence();
+#pragma unroll
+            for (int tt = 0; tt < 16; ++tt) { exch[tt * 17 + t] = h0[tt]; exch1[tt * 17 + t] = h1[tt]; }
+            wave_lds_fence();
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { e0[r] = exch[t * 17 + r]; e1[r] = exch1[t * 17 + r]; }
+            inv_pass2_lds(e0, twrow, y0);
+            inv_pass2_lds(e1, twrow, y1);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, y0[i]);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) store_streaming(dst + (long)S * DY + 16 * i, y1[i]);
+        } else {
+            // lane t = r + 8 h finishes channel h: modes r + 8 c; even c come from lanes t < 8, odd c from lanes t >= 8
+            cpx c8[8];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const cpx got = rotate8(upper ? c0[a] : c1[a]);
+                c8[2 * a] = upper ? got : c0[a];
+                c8[2 * a + 1] = upper ? c1[a] : got;
+            }
+            rows128_backward(c8, twrow, exch, t, y0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                store_streaming(dst + 16 * i, y0[i]);
+                store_streaming(dst + (long)S * DY + 16 * i, y0[8 + i]);
+            }
         }
     }
 }
@@ -395,8 +564,8 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
             float2* dst = out + sigA * DY + t16;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                dst[16 * i] = yv[i];
-                if (hasB) dst[DY + 16 * i] = yv[8 + i];
+                store_streaming(dst + 16 * i, yv[i]);
+                if (hasB) store_streaming(dst + DY + 16 * i, yv[8 + i]);
             }
         }
         return;
@@ -421,7 +590,7 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
         group_backward<LOGDY>(c, tw, exch, t, yv);
         float2* dst = out + sig * DY + t;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[L * i] = yv[i];
+        for (int i = 0; i < 16; ++i) store_streaming(dst + L * i, yv[i]);
     }
     }
 }
@@ -467,21 +636,40 @@ static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const
     return hipGetLastError();
 }
 
-// algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks
+template <int LOGDY>
+static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                    hipStream_t stream)
+{
+    if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fused_fft_mfma_ifft_wave_kernel<LOGDY>, dim3((unsigned)(S * (N / 64))), dim3(64), 0, stream, (int)S, N, K,
+                       x, W, y, alpha);
+    return hipGetLastError();
+}
+
+// algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
+// 4 = as 2 with 32-channel output tiles (DY = 256), 5 = matrix cores, one wavefront per (signal set, output tile)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
     // by size (measured on MI355X):
     //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
     //    every K, even K = 8 where most of a chunk is padding;
-    //  * larger grids with K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
+    //  * grids of several items per SIMD: one wavefront per item (no barriers, nothing staged through LDS). At DY = 128
+    //    it is ahead for every K from about four items per CU; at DY = 256, where the block kernels are closer to
+    //    what the access pattern allows, from eight items per CU and not for 16 < K < 64;
+    //  * in between, K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
     //    its vector instructions there, up to half of which are the contraction;
-    //  * larger grids with K < 32: the SIMT kernel (three blocks per CU, no idle lanes in short chunks; a tie at K = 16).
-    int pick = algo == 4 ? 2 : algo;             // 4 = matrix cores, 512 threads, 32-channel tiles (DY = 256 only)
-    if (pick == 0) {
-        const bool built = logDY == 7 || logDY == 8;
-        pick = (built && S * (N / 64) <= cu_count()) ? 2 : (K >= 32 ? 3 : 1);
-    }
+    //  * in between, K < 32: the SIMT kernel (three blocks per CU, no idle lanes in short chunks; a tie at K = 16).
+    const bool built = logDY == 7 || logDY == 8;
+    const long items = S * (N / 64);
+    if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
+    if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
+    if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : 4) * (long)cu_count())
+        return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
+    if (algo == 0 && logDY == 8 && items >= 8L * cu_count() && (K <= 16 || K >= 64))
+        return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
+    int pick = algo == 4 ? 2 : algo;
+    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 ? 3 : 1);
     // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
         return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream);

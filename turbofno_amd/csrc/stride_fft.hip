@@ -136,7 +136,7 @@ __global__ __launch_bounds__(GeoStride<LOGDX>::THREADS) void ifft_stride_kernel(
     inv_pass2(e, tw, yv);
     float2* dst = out + (sig * DX + t) * DY + y;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dst[(long)L * i * DY] = yv[i];
+    for (int i = 0; i < 16; ++i) store_streaming(dst + (long)L * i * DY, yv[i]);
 }
 
 template <int LOGDX, bool INVERSE>
