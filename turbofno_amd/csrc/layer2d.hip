@@ -366,17 +366,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2*
 // i.e. three matrix instructions per 16 n x 16 m x 4 k instead of four: 25 % less matrix work, and the matrix work is
 // the part of this kernel that nothing overlaps with. Rows of a tile are 16 output channels n (not 8 x re|im); a wave
 // keeps the accumulators P1, P2, P3 of its four n tiles and stores a tile when its last chunk is done.
-// W'' tile in LDS: float4 {c, d - c, c + d, unused} at float index (k * kW3Row + n * 4): an operand fetch of 16 n for
-// one k is 256 contiguous bytes; rows of different k are padded by four floats so that the build (lanes along k) does
-// not put a whole wavefront on one bank.
-constexpr int kW3Row = 64 * 4 + 4;
+// W'' tile in LDS: three planes (c, d - c, c + d) of floats at index (k / 4) * kW3Group + (k % 4) * kW3Row + n.
+// An operand fetch (64 lanes: 4 k x 16 n) reads 16 consecutive floats of four rows 80 apart: one bank each. The
+// build's lanes run along k, the contiguous direction of W: a group stride of 1 (mod 64 banks) puts the 64 lanes of a
+// store on 64 different banks as well.
+constexpr int kW3Row = 80, kW3Group = 4 * kW3Row + 1, kW3Plane = (GEMM_KC / 4) * kW3Group;
 
 template <int NG, bool MULTI>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float2* __restrict__ A,
                                                                      const float2* __restrict__ W, float2* __restrict__ C,
                                                                      long Mtot, int N, int K, float2 alpha, float2 beta)
 {
-    extern __shared__ float sW[];                     // GEMM_KC * kW3Row floats
+    extern __shared__ float sW[];                     // 3 * kW3Plane floats
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.y * 64;
     const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
@@ -418,7 +419,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
             const int idx = tid + u * GEMM_THREADS;
             const int k = idx % KCH, n = idx / KCH;
             const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
-            *reinterpret_cast<float4*>(&sW[k * kW3Row + n * 4]) = make_float4(c, d - c, c + d, 0.f);
+            float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
+            dstw[0] = c;
+            dstw[kW3Plane] = d - c;
+            dstw[2 * kW3Plane] = c + d;
         }
         if constexpr (MULTI) {
 #pragma unroll
@@ -430,13 +434,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if constexpr (!MULTI) p1[t] = p2[t] = p3[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
-            const float* wrow = &sW[kq * kW3Row + (t * 16 + col) * 4];
+            const float* wrow = &sW[kq * kW3Row + t * 16 + col];
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
-                const float4 w = *reinterpret_cast<const float4*>(wrow + g * 4 * kW3Row);
-                p1[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.x, bv[g].x + bv[g].y, p1[t], 0, 0, 0);
-                p2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.y, bv[g].x, p2[t], 0, 0, 0);
-                p3[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w.z, bv[g].y, p3[t], 0, 0, 0);
+                const float* w = wrow + g * kW3Group;
+                p1[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0], bv[g].x + bv[g].y, p1[t], 0, 0, 0);
+                p2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[kW3Plane], bv[g].x, p2[t], 0, 0, 0);
+                p3[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * kW3Plane], bv[g].y, p3[t], 0, 0, 0);
             }
             if (last) {
                 // D[row = 4 kq + v][col]: output channel n0 + 16 t + 4 kq + v, column m = wave * 16 + col
@@ -522,7 +526,7 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
     // more than 16 channels: three real products per complex one (25 % less matrix work); K <= 16 is bound by the
     // tile build and the stores, where the four-product kernel is slightly faster
     if (K > 16) {
-        constexpr size_t bytes3 = sizeof(float) * GEMM_KC * kW3Row;
+        constexpr size_t bytes3 = sizeof(float) * 3 * kW3Plane;
         auto launch3 = [&](auto ng_const, auto multi_const) -> hipError_t {
             constexpr int NG = decltype(ng_const)::value;
             constexpr bool MULTI = decltype(multi_const)::value;
