@@ -5,8 +5,8 @@
 
 namespace tfno {
 
-// LDS layout of a real-expanded W' tile for v_mfma_f32_16x16x4_f32 (shared by cgemm_modes_kernel and the matrix-core
-// 1D kernel): float index  (k/4)*kWGroup + ((k&3)>>1)*kWHalf + n'*4 + (k&1)*2 + c  holds W'[n' = 2n + c'][2k + c],
+// LDS layout of a real-expanded W' tile for v_mfma_f32_16x16x4_f32 (the block-per-item matrix-core
+// 1D kernels): float index  (k/4)*kWGroup + ((k&3)>>1)*kWHalf + n'*4 + (k&1)*2 + c  holds W'[n' = 2n + c'][2k + c],
 // {Wr, -Wi} for c' = 0 and {Wi, Wr} for c' = 1. An operand read (16 n' x 4 channels) takes 256 contiguous bytes per
 // half wavefront: conflict free. The strides are 512 + 4 and 1024 + 8 floats so that the tile BUILD, whose lanes run
 // along k (the contiguous direction of W in memory), spreads a half wavefront over all 64 banks as well; with the

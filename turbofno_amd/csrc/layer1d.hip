@@ -169,8 +169,8 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
 //     first pass has consumed it), so they travel under the exchanges, the W tile builds and the matrix work;
 //   * C'[n'][m] += W'[n'][k'] A'[k'][m] is the 4-real form of the complex product on v_mfma_f32_16x16x4_f32:
 //     n' = (n, re|im) 128 rows, m 64 columns = 8 x 4 tiles, four per wave (one m tile, four n' tiles), so one read of
-//     A from LDS feeds eight matrix instructions. W' (alpha folded in) uses the conflict-free LDS order of
-//     cgemm_modes_kernel; sA has a pitch of 80 complex so that the two k rows a half wave reads fall on disjoint banks;
+//     A from LDS feeds eight matrix instructions. W' (alpha folded in) uses the conflict-free LDS order kWGroup / kWHalf;
+//     sA has a pitch of 80 complex so that the two k rows a half wave reads fall on disjoint banks;
 //   * the product goes through LDS once (sC, pitch 72) to reach the lane groups that run the zero-padded backward
 //     transforms and store y.
 // sA aliases the exchange regions of the lane groups (the transforms of a chunk are complete before sA is written),

@@ -253,18 +253,22 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 
 // ---------------------------------------------------------------------------------------------
 // Mode-space complex GEMM on the fp32 matrix cores.
-//   C[n][m] = alpha * sum_k W[k + n*K] * A[k][m],   A: [K][Mtot], C: [N][Mtot]  (m contiguous)
+//   C[n][m] = alpha * sum_k W[k + n*K] * A[k][m] (+ beta C),   A: [K][Mtot], C: [N][Mtot]  (m contiguous)
 // Same contraction as the reference's cgemm / the GEMM phase of its fused kernel
-// (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4-205, operand layout lda=M, ldb=K, ldc=M),
-// expressed as the real product  [Cr;Ci] = [[Wr,-Wi],[Wi,Wr]] [Ar;Ai]  (4-real decomposition; for 16 < K <= 64 the
-// three-product form of cgemm_modes3m_kernel below is used instead) on
-// v_mfma_f32_16x16x4_f32: rows = (n, re/im), cols = 16 consecutive m, contraction = 4 channels x re|im.
-// A block is 16 waves; wave w owns the 16-m strip w and the whole 64-channel n tile (8 accumulators of
-// 16x16), so every element of A is loaded exactly once: the strip of a 64-channel chunk sits in 16 float2
-// registers per lane, all loads in flight while the W tile is built. One float2 of A feeds two matrix
-// instructions per n tile (real parts, then imaginary parts). The n tiles are the outer loop, so each is
-// stored as soon as it is complete and its stores drain under the matrix work of the next ones; the four
-// waves of a SIMD get descending priorities so that they run staggered.
+// (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4-205, operand layout lda=M, ldb=K, ldc=M), with three real
+// products per complex one instead of four:
+//   P1 = c (a + b),  P2 = (d - c) a,  P3 = (c + d) b   =>   re = P1 - P3,  im = P1 + P2      (alpha W = c + i d, A = a + i b)
+// i.e. three v_mfma_f32_16x16x4_f32 per 16 n x 16 m x 4 k: 25 % less matrix work than the real-expanded product, and
+// the matrix work is the part of this kernel that nothing overlaps with (all waves of the grid load, multiply and
+// store in step). Rows of a tile are 16 output channels n, columns 16 consecutive m, contraction 4 channels.
+// A block is 16 waves; wave w owns the 16-m strip w and the whole 64-channel n tile, so every element of A is loaded
+// exactly once: the strip of a chunk sits in NG float2 registers per lane, all loads in flight while the W tile is
+// built. The n tiles are the outer loop, so each is stored as soon as it is complete and its stores drain under the
+// matrix work of the next ones.
+//   NG    = channel groups of four per chunk that can hold data (4, 8, 12, 16 for K <= 16, 32, 48, 64): a template
+//           parameter so that the loops stay unrolled and no loads or matrix work are spent on zero padding;
+//   MULTI = K > 64: chunks of 4 NG = 32 channels with the twelve accumulator tiles of a wave kept across them
+//           (125 registers; 64-channel chunks would spill); otherwise one chunk and transient accumulators.
 // ---------------------------------------------------------------------------------------------
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -272,100 +276,6 @@ constexpr int GEMM_KC = 64;         // channels per LDS-resident W chunk
 constexpr int GEMM_THREADS = 1024;  // 16 waves x 16 m
 constexpr int GEMM_MBLOCK = 256;    // m per block
 
-// NG = channel groups of four per chunk that can hold data: 16 in general; 4, 8 or 12 for K <= 16, 32, 48, where the
-// single chunk then does no loads and no matrix work on zero padding. A template parameter so that the loops stay
-// unrolled and branch free.
-template <int NG>
-__global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes_kernel(const float2* __restrict__ A,
-                                                                   const float2* __restrict__ W, float2* __restrict__ C,
-                                                                   long Mtot, int N, int K, float2 alpha, float2 beta)
-{
-    // sW[(k/4)*kWGroup + ((k&3)>>1)*kWHalf + n'*4 + (k&1)*2 + c] = Wreal[n' = 2 n + c'][k' = 2 k + c]:
-    // {Wr, -Wi} for c'=0, {Wi, Wr} for c'=1. In one operand read (16 n' x 4 channels) lanes 0-31 cover 256
-    // contiguous bytes in lane order pairs and lanes 32-63 the next 256: no bank conflicts.
-    extern __shared__ float sW[];                     // (GEMM_KC / 4) * kWGroup floats
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
-    const int n0 = blockIdx.y * 64;
-    switch (wave >> 2) {                      // waves w, w+4, w+8, w+12 share a SIMD
-    case 0: __builtin_amdgcn_s_setprio(3); break;
-    case 1: __builtin_amdgcn_s_setprio(2); break;
-    case 2: __builtin_amdgcn_s_setprio(1); break;
-    default: __builtin_amdgcn_s_setprio(0); break;
-    }
-
-    floatx4 acc[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) acc[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
-
-    // scalar base per k group + one 32-bit lane offset keeps the addresses out of the vector registers
-    const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
-    const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
-    const bool active = (long)blockIdx.x * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
-    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
-    const unsigned out_off = (unsigned)(2 * kq * Mtot) + (unsigned)(wave * 16 + col);
-    const bool has_beta = beta.x != 0.f || beta.y != 0.f;
-
-    for (int kc = 0; kc < K; kc += GEMM_KC) {
-        const int kn = (K - kc) < GEMM_KC ? (K - kc) : GEMM_KC;   // multiple of 8 (caller contract)
-        const bool last = kc + GEMM_KC >= K;
-        // the wave's whole A strip of this chunk: lane (kq, col) holds channels kc + 4 g + kq, g = 0..15
-        float2 bv[NG];
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-            bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
-        __syncthreads();
-        // W tile: lanes run along k, the contiguous direction of W[k + n*K], so a wave reads 512 contiguous bytes
-        constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
-        float2 wv[WPT];
-#pragma unroll
-        for (int u = 0; u < WPT; ++u) {
-            const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
-            wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
-        }
-#pragma unroll
-        for (int u = 0; u < WPT; ++u) {
-            const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
-            const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
-            float* dstw = &sW[(k >> 2) * kWGroup + ((k & 3) >> 1) * kWHalf + (2 * n) * 4 + (k & 1) * 2];
-            *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
-            *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
-        }
-        __syncthreads();
-        if (!active) continue;
-        // n tile outermost: a tile is complete after its 2 * kn / 4 matrix instructions and, in the last chunk, is
-        // stored at once, so its stores drain under the matrix work of the following tiles
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const float* wrow = &sW[(kq >> 1) * kWHalf + (t * 16 + col) * 4 + (kq & 1) * 2];
-#pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                const float2 a = *reinterpret_cast<const float2*>(wrow + g * kWGroup);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, bv[g].x, acc[t], 0, 0, 0);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, bv[g].y, acc[t], 0, 0, 0);
-            }
-            if (last) {
-                // D[row = 4 kq + v][col]: row n' = 16 t + 4 kq + v = 2 n_local + c'  ->  n_local = 8 t + 2 kq + (v >> 1)
-                float2* p0 = cblk + (long)(n0 + 8 * t) * Mtot + out_off;
-                float2* p1 = cblk + (long)(n0 + 8 * t + 1) * Mtot + out_off;
-                float2 r0 = make_float2(acc[t][0], acc[t][1]), r1 = make_float2(acc[t][2], acc[t][3]);
-                if (has_beta) {          // C = alpha A W + beta C (the reference's cgemm / variant B)
-                    r0 = cadd(r0, cmul(*p0, beta));
-                    r1 = cadd(r1, cmul(*p1, beta));
-                }
-                *p0 = r0;                // plain stores: the backward kernel reads C back through the caches
-                *p1 = r1;
-            }
-        }
-    }
-}
-
-// The same contraction with three real products per complex one instead of four:
-//   P1 = c (a + b),  P2 = (d - c) a,  P3 = (c + d) b   =>   re = P1 - P3,  im = P1 + P2      (W' = c + i d, A = a + i b)
-// i.e. three matrix instructions per 16 n x 16 m x 4 k instead of four: 25 % less matrix work, and the matrix work is
-// the part of this kernel that nothing overlaps with. Rows of a tile are 16 output channels n (not 8 x re|im); a wave
-// keeps the accumulators P1, P2, P3 of its four n tiles and stores a tile when its last chunk is done.
 // W'' tile in LDS: three planes (c, d - c, c + d) of floats at index (k / 4) * kW3Group + (k % 4) * kW3Row + n.
 // An operand fetch (64 lanes: 4 k x 16 n) reads 16 consecutive floats of four rows 80 apart: one bank each. The
 // build's lanes run along k, the contiguous direction of W: a group stride of 1 (mod 64 banks) puts the 64 lanes of a
@@ -513,37 +423,23 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
 {
     if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
-    constexpr size_t lds_bytes = sizeof(float) * (GEMM_KC / 4) * kWGroup;      // 66,048 B: above the static limit
-    auto launch = [&](auto ng_const) -> hipError_t {
+    constexpr size_t lds_bytes = sizeof(float) * 3 * kW3Plane;      // 61,632 B: above the static limit
+    auto launch = [&](auto ng_const, auto multi_const) -> hipError_t {
         constexpr int NG = decltype(ng_const)::value;
+        constexpr bool MULTI = decltype(multi_const)::value;
         static std::atomic<unsigned long long> served;
-        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes_kernel<NG>), lds_bytes, served);
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_kernel<NG, MULTI>), lds_bytes, served);
             e != hipSuccess)
             return e;
-        hipLaunchKernelGGL(cgemm_modes_kernel<NG>, grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K, alpha, beta);
+        hipLaunchKernelGGL((cgemm_modes3m_kernel<NG, MULTI>), grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K,
+                           alpha, beta);
         return hipGetLastError();
     };
-    // more than 16 channels: three real products per complex one (25 % less matrix work); K <= 16 is bound by the
-    // tile build and the stores, where the four-product kernel is slightly faster
-    if (K > 16) {
-        constexpr size_t bytes3 = sizeof(float) * 3 * kW3Plane;
-        auto launch3 = [&](auto ng_const, auto multi_const) -> hipError_t {
-            constexpr int NG = decltype(ng_const)::value;
-            constexpr bool MULTI = decltype(multi_const)::value;
-            static std::atomic<unsigned long long> served3;
-            if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_kernel<NG, MULTI>), bytes3, served3);
-                e != hipSuccess)
-                return e;
-            hipLaunchKernelGGL((cgemm_modes3m_kernel<NG, MULTI>), grid, dim3(GEMM_THREADS), bytes3, stream, A, W, C, Mtot, N, K,
-                               alpha, beta);
-            return hipGetLastError();
-        };
-        if (K <= 32) return launch3(std::integral_constant<int, 8>{}, std::false_type{});
-        if (K <= 48) return launch3(std::integral_constant<int, 12>{}, std::false_type{});
-        if (K <= GEMM_KC) return launch3(std::integral_constant<int, 16>{}, std::false_type{});
-        return launch3(std::integral_constant<int, 8>{}, std::true_type{});
-    }
-    return launch(std::integral_constant<int, 4>{});
+    if (K <= 16) return launch(std::integral_constant<int, 4>{}, std::false_type{});
+    if (K <= 32) return launch(std::integral_constant<int, 8>{}, std::false_type{});
+    if (K <= 48) return launch(std::integral_constant<int, 12>{}, std::false_type{});
+    if (K <= GEMM_KC) return launch(std::integral_constant<int, 16>{}, std::false_type{});
+    return launch(std::integral_constant<int, 8>{}, std::true_type{});
 }
 
 }  // namespace tfno
