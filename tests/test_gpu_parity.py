@@ -65,6 +65,24 @@ def test_layer_1d_both_contractions(bs, DY, K, N, alpha, algo, tol, monkeypatch)
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d algo %d" % algo)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_layer_1d_random_shapes(seed, tol, monkeypatch):
+    """seeded random shapes (odd S, three N tiles, K up to 136, complex alpha) through every 1D kernel choice"""
+    rng = np.random.default_rng(1000 + seed)
+    DY = int(rng.choice([128, 256]))
+    K = 8 * int(rng.integers(1, 18))
+    N = 64 * int(rng.integers(1, 4))
+    S = int(rng.integers(1, 41))
+    algo = seed % 6
+    alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
+    print("case layer_1d random", seed, "S", S, "DY", DY, "K", K, "N", N, "algo", algo, flush=True)
+    monkeypatch.setenv("TURBOFNO_1D_ALGO", str(algo))
+    x, W = workloads.uniform_1d(seed, S, DY, K, N)
+    y = tf.layer_1d(dev(x), dev(W), alpha=alpha)
+    torch.cuda.synchronize()
+    check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d random %d" % seed)
+
+
 @pytest.mark.parametrize("bs,DY,K,N", [
     (1030, 128, 16, 64),             # DY=128: from two items per CU on for K <= 16
     (600, 128, 40, 128),             # DY=128, 1200 items, K = 5 rounds of 8 channels
