@@ -145,6 +145,23 @@ def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     check(y, oracle.layer_2d(x, W, alpha), tol, "layer_2d algo=%d" % algo)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_layer_2d_random_shapes(seed, tol):
+    """seeded random 2D shapes through the size rule, the three-kernel path and the whole-image path"""
+    rng = np.random.default_rng(2000 + seed)
+    DX, DY = int(rng.choice([128, 256])), int(rng.choice([128, 256]))
+    K = 8 * int(rng.integers(1, 12))
+    N = 64 * int(rng.integers(1, 3))
+    bs = int(rng.integers(1, 4))
+    algo = seed % 3
+    alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
+    print("case layer_2d random", seed, "bs", bs, DX, DY, "K", K, "N", N, "algo", algo, flush=True)
+    x, W = workloads.uniform_2d(seed, bs, DX, DY, K, N)
+    y = tf.layer_2d(dev(x), dev(W), alpha=alpha, algo=algo)
+    torch.cuda.synchronize()
+    check(y, oracle.layer_2d(x, W, alpha), tol, "layer_2d random %d" % seed)
+
+
 def test_layer_2d_closed_forms(tol):
     """impulse and in-band tone through the whole-image path (analytic expectations, no oracle)."""
     K, bs, D, N = 8, 1, 256, 64
