@@ -46,7 +46,7 @@ def test_layer_1d(bs, DY, K, N, alpha, tol):
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d")
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("bs,DY,K,N,alpha", [
     (2, 256, 32, 64, 1.0),           # exactly one chunk of the matrix-core kernel
     (3, 256, 72, 128, 1 - 1j),       # chunks 32 + 32 + 8, two N tiles

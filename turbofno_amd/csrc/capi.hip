@@ -71,12 +71,13 @@ const char* turbofno_last_error_string(void) { return g_err; }
 // The fused 1D entry point keeps the reference's kernel signature, which has no room for an algorithm selector:
 // TURBOFNO_1D_ALGO in the environment (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with 512- / 256-thread
 // blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one wavefront per signal
-// set and output tile) overrides the choice.
+// set and output tile, 6 matrix cores with the K channels of an item split over the waves of a block) overrides the
+// choice.
 static int algo_1d()
 {
     const char* e = getenv("TURBOFNO_1D_ALGO");
     const int a = e ? atoi(e) : 0;
-    return (a >= 1 && a <= 5) ? a : 0;
+    return (a >= 1 && a <= 6) ? a : 0;
 }
 
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,

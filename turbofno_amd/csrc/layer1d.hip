@@ -519,6 +519,101 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
 }
 
+// Fused 1D layer for small grids (every block has a CU to itself), DY = 256: the eight waves of a block share ONE
+// item (signal set, 32 output channels) and split its K input channels. Operands as in the one-wavefront kernel above:
+// wave w transforms channels 32 r + 4 w + g in round r and multiplies them straight out of its registers into its own
+// partial accumulators (4 n' tiles x 4 m tiles), so the K loop has no barrier and stages nothing through LDS. The
+// eight partial products meet in LDS once (sP[w][n][m], pitch 72 complex: conflict-free b64 stores), every lane group
+// sums the eight partials of one output channel and runs its backward transform. The chain of latencies of an item
+// is K / 32 rounds + one reduction + one backward pass, against three barriers and two tile builds per 32 channels
+// in the kernel that shares the spectra through LDS.
+constexpr int SPLIT_NT = 32, SPLIT_PP = 72;
+constexpr size_t SPLIT_LDS = sizeof(float2) * 8 * SPLIT_NT * SPLIT_PP;       // 147,456 B; covers the 32 exchange regions
+
+__global__ __launch_bounds__(512) void fused_fft_mfma_ifft_split_kernel(int S, int N, int K, const float2* __restrict__ x,
+                                                                        const float2* __restrict__ W, float2* __restrict__ y,
+                                                                        float2 alpha)
+{
+    constexpr int DY = 256, EXCH = 16 * 17;
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, t = lane & 15;
+    float2* exch = lds + (4 * w + g) * EXCH;                      // the partials overlay these after the K loop
+    long s;
+    int ntile;
+    decode_block_1d(S, N / SPLIT_NT, s, ntile);
+    const int n0 = ntile * SPLIT_NT;
+    const bool odd = t & 1;
+    cpx tw[16];
+    load_lane_twiddles<8>(t, tw);
+
+    floatx4_1d acc[4][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) acc[nt][a] = floatx4_1d{ 0.f, 0.f, 0.f, 0.f };
+
+    // K is a multiple of 8 and a wave covers four consecutive channels: a wave is either fully inside K or idle
+    const int k0 = 4 * w + g;
+    const float2* src = x + ((long)k0 * S + s) * DY + t;
+    const float2* wsrc = W + k0 + (long)(n0 + (t >> 1)) * K;      // W[k][n = n0 + 8 nt + t / 2]
+    auto issue = [&](cpx (&dst)[16], int kc) {                    // samples t + 16 i of channel kc + k0
+        const float2* p = src + (long)kc * S * DY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[i] = p[16 * i];
+    };
+    // the buffer is refilled as soon as the first pass has consumed it (a second buffer, two rounds ahead, was
+    // measured slower: a round is bound by its arithmetic, not by the latency of its loads)
+    auto round = [&](cpx (&v)[16], int kc) {
+        float2 wv[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) wv[nt] = wsrc[kc + (long)(8 * nt) * K];
+        cpx gg[16], out[4];
+        fwd_pass1(v, tw, gg);
+        if (kc + 32 + 4 * w < K) issue(v, kc + 32);
+        group_forward_finish<8>(gg, exch, t, out);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            const float2 wa = make_float2(wv[nt].x * alpha.x - wv[nt].y * alpha.y, wv[nt].x * alpha.y + wv[nt].y * alpha.x);
+            const float ax = odd ? wa.y : wa.x, ay = odd ? wa.x : -wa.y;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                acc[nt][a] = __builtin_amdgcn_mfma_f32_16x16x4f32(ax, out[a].x, acc[nt][a], 0, 0, 0);
+                acc[nt][a] = __builtin_amdgcn_mfma_f32_16x16x4f32(ay, out[a].y, acc[nt][a], 0, 0, 0);
+            }
+        }
+    };
+    cpx v[16];
+    if (4 * w < K) issue(v, 0);
+    for (int kc = 0; kc + 4 * w < K; kc += 32) round(v, kc);
+    __syncthreads();                                              // every wave is done with its exchange regions
+    // D[row = 4 g + v][column = t] of tile (nt, a): channel n = 8 nt + 2 g + (v >> 1), re | im = v & 1, mode t + 16 a
+    float2* sP = lds + (long)w * SPLIT_NT * SPLIT_PP;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            sP[(8 * nt + 2 * g) * SPLIT_PP + t + 16 * a] = make_float2(acc[nt][a][0], acc[nt][a][1]);
+            sP[(8 * nt + 2 * g + 1) * SPLIT_PP + t + 16 * a] = make_float2(acc[nt][a][2], acc[nt][a][3]);
+        }
+    __syncthreads();
+    // lane group (w, g) owns output channel n = 4 w + g: sum of the eight partials, modes t + 16 a
+    const int n = 4 * w + g;
+    cpx c[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        cpx sum = lds[n * SPLIT_PP + t + 16 * a];
+#pragma unroll
+        for (int ww = 1; ww < 8; ++ww) sum = cadd(sum, lds[(ww * SPLIT_NT + n) * SPLIT_PP + t + 16 * a]);
+        c[a] = sum;
+    }
+    __syncthreads();                                              // the partials are consumed: exchange regions again
+    cpx yv[16];
+    group_backward<8>(c, tw, exch, t, yv);
+    float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, yv[i]);
+}
+
 // Stand-alone truncated forward / zero-padded backward transforms of contiguous signals (variants A, B, C):
 //   fft_stride_DY : in[nsig][DY] -> out[nsig][64]      ifft_stride_DY : in[nsig][64] -> out[nsig][DY]
 // Replace fft_N_stride_DY / ifft_N_stride_DY of the missing TurboFFT submodule (launched at
@@ -647,7 +742,8 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
 }
 
 // algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
-// 4 = as 2 with 32-channel output tiles (DY = 256), 5 = matrix cores, one wavefront per (signal set, output tile)
+// 4 = as 2 with 32-channel output tiles (DY = 256), 5 = matrix cores, one wavefront per (signal set, output tile),
+// 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
@@ -670,6 +766,18 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 ? 3 : 1);
+    // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
+    // shares the spectra through LDS; level at K = 32)
+    if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cu_count()))) {
+        static std::atomic<unsigned long long> served;
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_split_kernel), SPLIT_LDS, served);
+            e != hipSuccess)
+            return e;
+        if (S * (N / SPLIT_NT) > 0x7fffffffL) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(fused_fft_mfma_ifft_split_kernel, dim3((unsigned)(S * (N / SPLIT_NT))), dim3(512), SPLIT_LDS, stream,
+                           (int)S, N, K, x, W, y, alpha);
+        return hipGetLastError();
+    }
     // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
         return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream);
