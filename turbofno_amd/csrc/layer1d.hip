@@ -380,11 +380,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     constexpr int DY = 1 << LOGDY, EXCH = 16 * 17;
     constexpr bool PAIR = LOGDY == 7;
     constexpr int CH = PAIR ? 8 : 4;                              // channels per round
-    __shared__ float2 lds[8 * EXCH + kTwLdsSize];
+    constexpr int REGIONS = PAIR ? 4 : 8;                         // DY = 256: a second set for the paired backward transforms
+    __shared__ float2 lds[REGIONS * EXCH + kTwLdsSize];
     const int lane = threadIdx.x, g = lane >> 4, t = lane & 15;
     float2* exch = lds + g * EXCH;
-    float2* exch1 = exch + 4 * EXCH;                              // second region: two backward transforms in flight
-    float2* twtab = lds + 8 * EXCH;
+    float2* exch1 = exch + (PAIR ? 0 : 4 * EXCH);                 // second region: two backward transforms in flight
+    float2* twtab = lds + REGIONS * EXCH;
     fill_lds_twiddles<LOGDY>(twtab, lane, 64);
     const float2* twrow = twtab + t * kTwLdsPitch;
     __syncthreads();
