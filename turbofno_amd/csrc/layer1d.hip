@@ -193,7 +193,8 @@ template <int LOGDY, int THREADS_, int NT_ = 64> struct GeoMfma1D {
     static constexpr int WTILE = (KC / 4) * kWGroup / 2;                                   // W' tile in complex units
     static constexpr int REGION1 = COMPACT ? WTILE : (WTILE > NT * PC ? WTILE : NT * PC);  // W' | sC   (complex)
     static_assert(!COMPACT || NT * PC <= REGION0, "sC must fit the exchange regions");
-    static_assert(NT == 64 || (NT == 32 && THREADS_ == 512 && LOGDY == 8), "32-channel tiles: DY = 256, 512 threads");
+    static_assert(NT == 64 || (NT == 32 && THREADS_ == 512), "32-channel tiles: 512 threads");
+    static constexpr int PASSES = (NT + KC - 1) / KC;         // backward passes; the last may use only NT % KC lane groups
     static constexpr int TWTAB = COMPACT ? kTwLdsSize : 0;    // compact: twiddles in LDS instead of 30 registers
     static constexpr int DEPTH = COMPACT ? 1 : 2;             // chunks of loads in flight per lane group
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1 + TWTAB);
@@ -325,15 +326,16 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     __syncthreads();
     // every pass takes its modes before the first backward transform: in the compact layout the exchange regions
     // overlay sC
-    cpx c[NT / KC][MM];
+    cpx c[G::PASSES][MM];
 #pragma unroll
-    for (int pass = 0; pass < NT / KC; ++pass)
+    for (int pass = 0; pass < G::PASSES; ++pass)
 #pragma unroll
-        for (int a = 0; a < MM; ++a) c[pass][a] = sC[(g + KC * pass) * PC + t + L * a];
+        for (int a = 0; a < MM; ++a) c[pass][a] = (g + KC * pass < NT) ? sC[(g + KC * pass) * PC + t + L * a] : make_float2(0.f, 0.f);
     if constexpr (G::COMPACT) __syncthreads();
 #pragma unroll
-    for (int pass = 0; pass < NT / KC; ++pass) {
+    for (int pass = 0; pass < G::PASSES; ++pass) {
         const int n = g + KC * pass;
+        if (n >= NT) break;                                    // whole waves (NT and KC are multiples of 32 channels)
         cpx yv[16];
         if constexpr (PAIR) {
             pair128_backward(c[pass], tw, exch, t16, yv);
@@ -743,7 +745,7 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
 }
 
 // algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
-// 4 = as 2 with 32-channel output tiles (DY = 256), 5 = matrix cores, one wavefront per (signal set, output tile),
+// 4 = as 2 with 32-channel output tiles, 5 = matrix cores, one wavefront per (signal set, output tile),
 // 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
@@ -783,6 +785,8 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
         return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream);
     if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 2 && logDY == 7 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
+        return launch_fused_mfma<7, 512, 32>(S, N, K, x, W, y, alpha, stream);
     if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream);
     if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream);
     if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream);
