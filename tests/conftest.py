@@ -31,5 +31,5 @@ def max_rel(a, b):
 
 @pytest.fixture(scope="session")
 def tol():
-    # BASELINE north_star: relative L2 <= 1e-5, max element relative error <= 1e-4 in complex fp32
+    # parity bar of this path: relative L2 <= 1e-5, max element relative error <= 1e-4 in complex fp32
     return {"l2": 1e-5, "max": 1e-4}
