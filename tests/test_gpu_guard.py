@@ -65,7 +65,7 @@ def test_cgemm_stays_in_bounds(M, N, K):
     assert float(torch.linalg.vector_norm(C - ref) / torch.linalg.vector_norm(ref)) <= 1e-5
 
 
-@pytest.mark.parametrize("D,other,nsig", [(128, 48, 3), (256, 16, 5), (512, 32, 2), (1024, 16, 1)])
+@pytest.mark.parametrize("D,other,nsig", [(128, 48, 3), (256, 16, 5), (512, 32, 2), (1024, 16, 1), (256, 96, 3), (128, 64, 2)])
 def test_stride_kernels_stay_in_bounds(D, other, nsig):
     print("guard stride", D, other, nsig, flush=True)
     rng = np.random.default_rng(D)
