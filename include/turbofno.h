@@ -129,6 +129,18 @@ int turbofno_fused_fft_cgemm(int logDY, long M, int N, int K, const void* x, con
 int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, const void* W, void* C, void* y,
                               float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
 
+/*
+ * Process-wide choice of the fused 1D kernel behind turbofno_fused_fft_cgemm_ifft / turbofno_layer_1d and the Y stage
+ * of the three-kernel 2D path (their reference-shaped signatures have no room for a selector): 0 = by problem size
+ * (default), 1 = SIMT contraction, 2 / 3 = matrix cores with 512- / 256-thread blocks, 4 = matrix cores, 512 threads,
+ * 32-channel output tiles, 5 = matrix cores, one wavefront per signal set and output tile, 6 = matrix cores, the K
+ * channels of an item split over the waves of a block. A value a kernel is not built for falls back to the choice by
+ * size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
+ */
+#define TURBOFNO_1D_ALGO_MAX 6
+int turbofno_set_1d_algo(int algo);
+int turbofno_get_1d_algo(void);
+
 /* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
 const char* turbofno_last_error_string(void);
 

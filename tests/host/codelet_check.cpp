@@ -1,8 +1,13 @@
-// CPU check of the register FFT codelets (turbofno_amd/csrc/fft_codelets.h built with
-// TFNO_HOST_CHECK): emulates the lanes of one L-lane group in a loop, performs the exchange as a
+// CPU check of the register FFT codelets (turbofno_amd/csrc/fft_codelets.h compiled by the host compiler, with
+// the vector types and function qualifiers supplied here): emulates the lanes of one L-lane group in a loop, performs the exchange as a
 // plain matrix transpose, and compares the truncated forward / zero-padded backward transform of
 // random data against a double-precision O(D^2) DFT. Prints "OK" and exits 0 on success.
-#define TFNO_HOST_CHECK
+#include <cmath>
+struct float2 { float x, y; };
+struct alignas(16) float4 { float x, y, z, w; };
+static inline float2 make_float2(float x, float y) { return float2{ x, y }; }
+#define TFNO_DEV static inline
+#define TFNO_TABLE static const
 #include "../../turbofno_amd/csrc/fft_codelets.h"
 #include <complex>
 #include <cstdio>

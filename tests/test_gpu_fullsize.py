@@ -1,9 +1,11 @@
 """GPU checks at the full sizes of the benchmark configurations.
 
-Where the CPU oracle finishes in seconds (all 1D configurations) the HIP path is compared with it directly; at the
-2D sizes it is compared with an independent library evaluation on the GPU (rocFFT through torch.fft plus a torch
-contraction, complex64) and through properties that do not depend on size: linearity in x, agreement of the two
-independent 2D algorithms, and idempotence of the layer when it is a pure low-pass projection.
+Where the CPU oracle finishes in seconds (all 1D configurations) the HIP path is compared with it directly. At the
+2D sizes batch elements are independent, so the full-size run on the GPU is compared with the oracle on slices:
+y[:, b] against oracle.layer_2d(x[:, b:b+1], W) for a few b. In addition it is compared with an independent library
+evaluation on the GPU (rocFFT through torch.fft plus a torch contraction, complex64) and through properties that do
+not depend on size: linearity in x, agreement of the two independent 2D algorithms, and idempotence of the layer when
+it is a pure low-pass projection.
 """
 import numpy as np
 import pytest
@@ -12,7 +14,7 @@ import torch
 import oracle
 import turbofno_amd as tf
 from turbofno_amd import workloads
-from conftest import max_rel, rel_l2
+from conftest import max_rel, max_rel_elementwise, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -50,10 +52,10 @@ def test_config2_sweep_against_oracle(tol):
 
 @pytest.mark.parametrize("K", [64, 128])
 @pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6])
-def test_config3_large_hidden_against_oracle(K, algo, tol, monkeypatch):
+def test_config3_large_hidden_against_oracle(K, algo, tol, algo_1d):
     """1D bs=64, DY=256, N=128, K in {64, 128}, smooth input: size-chosen kernel, SIMT kernel, the three matrix-core variants"""
     print("config3", K, algo, flush=True)
-    monkeypatch.setenv("TURBOFNO_1D_ALGO", str(algo))
+    algo_1d(algo)
     x, W = workloads.smooth_1d(0x5EED + 3, 64, 256, K, 128)
     y = tf.layer_1d(torch.from_numpy(x).cuda(), torch.from_numpy(W).cuda()).cpu().numpy()
     ref = oracle.layer_1d(x, W, 1.0)
@@ -79,6 +81,56 @@ def test_config4_grid_against_library(bs, D, K, tol):
 def headline():
     x_h, W_h = workloads.vorticity_2d(0x5EED + 5, 16, 256, 256, 64, 64)
     return torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
+
+
+def _check_batch_slices(y, x_h, W_h, alpha, batch_elements, tol, what):
+    """y[:, b] of a full-size GPU result against the fp64 oracle run on batch element b alone"""
+    for b in batch_elements:
+        ref = oracle.layer_2d(np.ascontiguousarray(x_h[:, b:b + 1]), W_h, alpha)
+        got = y[:, b:b + 1].cpu().numpy()
+        e2, em, ee = rel_l2(got, ref), max_rel(got, ref), max_rel_elementwise(got, ref)
+        print("%s b=%d rel_l2=%.3e max_rel=%.3e elementwise=%.3e" % (what, b, e2, em, ee), flush=True)
+        assert e2 <= tol["l2"] and em <= tol["max"] and ee <= tol["elem"], (what, b, e2, em, ee)
+
+
+@pytest.mark.parametrize("algo", [0, 1, 2])
+def test_headline_against_oracle_slices(algo, tol):
+    """configuration 5 (bs=16, 256 x 256, K=N=64, Gaussian random field) at full size; batch elements 0, 7, 15
+    against the oracle"""
+    print("headline vs oracle slices, algo", algo, flush=True)
+    x_h, W_h = workloads.vorticity_2d(0x5EED + 5, 16, 256, 256, 64, 64)
+    y = tf.layer_2d(torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda(), algo=algo)
+    torch.cuda.synchronize()
+    _check_batch_slices(y, x_h, W_h, 1.0, (0, 7, 15), tol, "headline algo %d" % algo)
+
+
+@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("K", [16, 32])
+def test_config4_bs16_against_oracle_slices(D, K, tol):
+    """configuration 4 at its largest batch, every algorithm, batch elements 0, 5, 15 against the oracle"""
+    x_h, W_h = workloads.uniform_2d(440 + D + K, 16, D, D, K, 64)
+    x, W = torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
+    for algo in (0, 1, 2):
+        print("config4 bs=16 vs oracle slices", D, K, "algo", algo, flush=True)
+        y = tf.layer_2d(x, W, alpha=1 - 1j, algo=algo)
+        torch.cuda.synchronize()
+        _check_batch_slices(y, x_h, W_h, 1 - 1j, (0, 5, 15), tol, "config4 D=%d K=%d algo %d" % (D, K, algo))
+
+
+@pytest.mark.parametrize("bs,DX,DY,K,N", [
+    (5, 256, 256, 64, 64),           # 320 input images on a 256-block persistent grid: 64 blocks take a second image
+    (9, 256, 256, 64, 128),          # 576 input and 1152 output images: up to three / five images per block
+    (11, 128, 256, 56, 64),          # 616 images of 128 x 256, K not a multiple of 16
+    (10, 256, 128, 64, 64),          # 640 images with paired rows of 128
+])
+def test_whole_image_persistent_loop_against_oracle(bs, DX, DY, K, N, tol):
+    """more images than persistent blocks, so that the image loop of the whole-image kernels and its look-ahead
+    loads across the image boundary run several times per block; a spread of batch elements against the oracle"""
+    print("whole-image persistent loop", bs, DX, DY, K, N, flush=True)
+    x_h, W_h = workloads.uniform_2d(900 + bs + DX + K, bs, DX, DY, K, N)
+    y = tf.layer_2d(torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda(), alpha=0.5 + 0.25j, algo=2)
+    torch.cuda.synchronize()
+    _check_batch_slices(y, x_h, W_h, 0.5 + 0.25j, sorted({0, 1, bs // 2, bs - 2, bs - 1}), tol, "persistent loop")
 
 
 def test_headline_against_library(headline, tol):

@@ -24,11 +24,11 @@ def intact(buf, what):
     assert bool((lo == CANARY).all()) and bool((hi == CANARY).all()), what + ": guard band overwritten"
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("bs,DY,K,N", [(3, 256, 72, 128), (5, 128, 40, 64), (1, 256, 8, 64), (7, 128, 136, 128)])
-def test_layer_1d_stays_in_bounds(bs, DY, K, N, algo, monkeypatch):
+def test_layer_1d_stays_in_bounds(bs, DY, K, N, algo, algo_1d):
     print("guard 1d", bs, DY, K, N, algo, flush=True)
-    monkeypatch.setenv("TURBOFNO_1D_ALGO", str(algo))
+    algo_1d(algo)
     x_h, W_h = workloads.uniform_1d(70 + bs + K, bs, DY, K, N)
     buf, y = guarded((N, bs, DY))
     tf.layer_1d(torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda(), y=y)

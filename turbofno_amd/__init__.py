@@ -23,6 +23,7 @@ from .api import (  # noqa: F401
     layer_2d_workspace_bytes,
     lib,
     library_path,
+    set_1d_algo,
 )
 
 ALGO_AUTO, ALGO_THREE_KERNEL, ALGO_WHOLE_IMAGE = 0, 1, 2

@@ -2,9 +2,9 @@
 // Declarations and the reference interfaces each entry point replaces are in include/turbofno.h.
 #include "../../include/turbofno.h"
 #include "kernels.h"
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 
 namespace {
 
@@ -69,16 +69,21 @@ int turbofno_abi_version(void) { return 1; }
 const char* turbofno_last_error_string(void) { return g_err; }
 
 // The fused 1D entry point keeps the reference's kernel signature, which has no room for an algorithm selector:
-// TURBOFNO_1D_ALGO in the environment (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with 512- / 256-thread
-// blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one wavefront per signal
-// set and output tile, 6 matrix cores with the K channels of an item split over the waves of a block) overrides the
-// choice.
-static int algo_1d()
+// the process-wide selector set by turbofno_set_1d_algo (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with
+// 512- / 256-thread blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one
+// wavefront per signal set and output tile, 6 matrix cores with the K channels of an item split over the waves of a
+// block) overrides the choice by size.
+static std::atomic<int> g_algo_1d{ 0 };
+static int algo_1d() { return g_algo_1d.load(std::memory_order_relaxed); }
+
+int turbofno_set_1d_algo(int algo)
 {
-    const char* e = getenv("TURBOFNO_1D_ALGO");
-    const int a = e ? atoi(e) : 0;
-    return (a >= 1 && a <= 6) ? a : 0;
+    if (algo < 0 || algo > TURBOFNO_1D_ALGO_MAX) return fail(TURBOFNO_ERR_INVALID_ARG, "1D algo %d outside 0..%d", algo, TURBOFNO_1D_ALGO_MAX);
+    g_algo_1d.store(algo, std::memory_order_relaxed);
+    return TURBOFNO_OK;
 }
+
+int turbofno_get_1d_algo(void) { return algo_1d(); }
 
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream)
@@ -212,14 +217,19 @@ size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, i
     return align256((size_t)K * bs * 64 * DY * sizeof(float2)) + align256((size_t)N * bs * 64 * DY * sizeof(float2));
 }
 
-int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y, float alpha_re,
-                      float alpha_im, void* workspace, size_t workspace_bytes, int algo, void* stream)
+// Both 2D entry points: validation, choice of algorithm, the three launches. `workspace` is the caller's buffer
+// (turbofno_layer_2d) or this GPU's copy of the static scratch array (turbofno_layer_2d_noalloc); `what` names it
+// in error messages.
+static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y, float alpha_re,
+                       float alpha_im, void* workspace, size_t workspace_bytes, const char* what, int algo, void* stream)
 {
     if (!x || !W || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "x, W and y must be non-null device pointers");
     if (bs <= 0) return fail(TURBOFNO_ERR_INVALID_ARG, "bs=%d must be positive", bs);
     int logDX = log2_exact(DX), logDY = log2_exact(DY);
     if (logDX < 0 || logDY < 0) return fail(TURBOFNO_ERR_INVALID_ARG, "DX=%d, DY=%d must be powers of two", DX, DY);
     if (int rc = check_gemm_dims((long)bs * 64 * 64, N, K)) return rc;
+    if ((long)K * bs > 0x7fffffffL || (long)N * bs > 0x7fffffffL)
+        return fail(TURBOFNO_ERR_INVALID_ARG, "K*bs=%ld or N*bs=%ld images exceed the grid limit", (long)K * bs, (long)N * bs);
     if (!length_built(logDX) || !length_built(logDY))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256, 512, 1024} are built", DX, DY);
     if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE)
@@ -229,23 +239,29 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     const int a = pick_algo(bs, DX, DY, K, algo);
     const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
     if (!workspace || workspace_bytes < need)
-        return fail(TURBOFNO_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need, workspace ? workspace_bytes : (size_t)0);
-    if ((size_t)workspace % 256) return fail(TURBOFNO_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+        return fail(TURBOFNO_ERR_WORKSPACE, "%s of %zu bytes required, %zu available", what, need, workspace ? workspace_bytes : (size_t)0);
+    if ((size_t)workspace % 256) return fail(TURBOFNO_ERR_WORKSPACE, "%s must be 256-byte aligned", what);
     hipStream_t st = (hipStream_t)stream;
     const float2 alpha = make_float2(alpha_re, alpha_im);
     char* ws = (char*)workspace;
     if (a == TURBOFNO_2D_WHOLE_IMAGE) {
         float2* spec = (float2*)ws;
         float2* cspec = (float2*)(ws + align256((size_t)K * bs * 4096 * sizeof(float2)));
-        if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, (long)K * bs, st), "fft2d_trunc launch")) return rc;
+        if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, K * bs, st), "fft2d_trunc launch")) return rc;
         if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, make_float2(0.f, 0.f), st), "cgemm_modes launch")) return rc;
-        return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, (long)N * bs, st), "ifft2d_pad launch");
+        return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, N * bs, st), "ifft2d_pad launch");
     }
     float2* t1 = (float2*)ws;
     float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));
     if (int rc = hip_status(tfno::launch_fft_stride(logDX, (const float2*)x, t1, DY, (long)K * bs, st), "fft_stride launch")) return rc;
     if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, algo_1d(), st), "fused_fft_cgemm_ifft launch")) return rc;
     return hip_status(tfno::launch_ifft_stride(logDX, t2, (float2*)y, DY, (long)N * bs, st), "ifft_stride launch");
+}
+
+int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y, float alpha_re,
+                      float alpha_im, void* workspace, size_t workspace_bytes, int algo, void* stream)
+{
+    return layer_2d_on(bs, DX, DY, K, N, x, W, y, alpha_re, alpha_im, workspace, workspace_bytes, "workspace", algo, stream);
 }
 
 }  // extern "C"

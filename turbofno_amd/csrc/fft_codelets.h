@@ -14,15 +14,9 @@
 //
 // DIR = -1 is the forward transform exp(-2 pi i jm/D); DIR = +1 the unnormalised backward one.
 #pragma once
-#ifdef TFNO_HOST_CHECK
-// Plain-C++ build of the same arithmetic for the CPU unit test of the codelets (no HIP runtime).
-#include <cmath>
-struct float2 { float x, y; };
-struct alignas(16) float4 { float x, y, z, w; };
-static inline float2 make_float2(float x, float y) { return float2{ x, y }; }
-#define TFNO_DEV static inline
-#define TFNO_TABLE static const
-#else
+// The arithmetic below is plain C++ over float2 / float4: a translation unit that is not compiled by hipcc (a CPU
+// unit test of the codelets) defines TFNO_DEV, TFNO_TABLE and those two vector types before including this header.
+#ifndef TFNO_DEV
 #include <hip/hip_runtime.h>
 #define TFNO_DEV __device__ __forceinline__
 #define TFNO_TABLE __device__ __constant__ const
@@ -243,7 +237,7 @@ template <int LOGD> TFNO_DEV void load_lane_twiddles(int t, cpx (&tw)[16])
 constexpr int kTwLdsPitch = 18;
 constexpr int kTwLdsSize = 16 * kTwLdsPitch;   // complex elements
 
-#ifndef TFNO_HOST_CHECK
+#ifdef __HIPCC__
 template <int LOGD> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
 {
     for (int e = tid; e < 256; e += nthreads) {      // all 16 lane rows (groups of fewer lanes use the first ones)
@@ -344,7 +338,7 @@ template <int L> TFNO_DEV void wide_backward_inputs(const cpx* exch, int t, cpx 
 // Orders LDS traffic of one wavefront: everything the wave wrote before is visible to its own
 // lanes after. DS operations of a wave complete in issue order, so no hardware wait is needed
 // beyond what the compiler inserts for the data dependency; this only stops compiler reordering.
-#ifndef TFNO_HOST_CHECK
+#ifdef __HIPCC__
 // Streaming (non-temporal) global accesses for data touched exactly once.
 typedef float tfno_v2f __attribute__((ext_vector_type(2)));
 TFNO_DEV cpx load_streaming(const cpx* p)

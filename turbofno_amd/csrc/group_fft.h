@@ -125,7 +125,7 @@ TFNO_DEV void group_backward_lds(const cpx (&c)[Geo1D<LOGD>::MM], const cpx* twr
 // each, so a group still moves 128 contiguous bytes per load or store. The first pass is a pair of 8-point FFTs;
 // after the exchange lane t = r + 8 h finishes row h: modes r + 8 c, c < 8. Twiddles w_128^(t r) come from the lane's
 // row of the LDS table.
-#ifndef TFNO_HOST_CHECK
+#ifdef __HIPCC__
 // g[0..7] / g[8..15]: first-pass results of row A / row B, already twiddled. On return out[c] = mode (t & 7) + 8 c
 // of row (t >> 3).
 TFNO_DEV void rows128_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&out)[8])

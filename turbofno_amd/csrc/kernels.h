@@ -50,9 +50,9 @@ hipError_t launch_fft_stride(int logDX, const float2* in, float2* out, int DY, l
 hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream);
 
 // Whole-image 2D path (DX, DY in {128, 256}): truncated 2D forward transform per image, mode-space CGEMM
-// on the matrix cores, zero-padded 2D backward transform per image.
-hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, long nimg, hipStream_t stream);
-hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, long nimg, hipStream_t stream);
+// on the matrix cores, zero-padded 2D backward transform per image. nimg: the C ABI rejects counts beyond INT_MAX.
+hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, int nimg, hipStream_t stream);
+hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, int nimg, hipStream_t stream);
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
                               float2 beta, hipStream_t stream);
 

@@ -699,6 +699,13 @@ static hipError_t launch_fused_1d(long S, int N, int K, const float2* x, const f
 {
     using G = Geo1D<LOGDY>;
     if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
+    if constexpr (G::LDS_BYTES > 64 * 1024) {          // DY = 128: 32 channels per chunk, 70 KiB
+        static std::atomic<unsigned long long> served;
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV>),
+                                             G::LDS_BYTES, served);
+            e != hipSuccess)
+            return e;
+    }
     dim3 grid((unsigned)(S * (N / 64)), 1, 1), block(256, 1, 1);
     hipLaunchKernelGGL((fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV>), grid, block, G::LDS_BYTES, stream, (int)S,
                        N, K, x, W, y, alpha, beta);
@@ -758,7 +765,8 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     //    what the access pattern allows, from eight items per CU and not for 16 < K < 64;
     //  * in between, K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
     //    its vector instructions there, up to half of which are the contraction;
-    //  * in between, K < 32: the SIMT kernel (three blocks per CU, no idle lanes in short chunks; a tie at K = 16).
+    //  * in between, K < 32: the SIMT kernel (three blocks per CU at DY = 256, two at DY = 128; no idle lanes in short
+    //    chunks; a tie at K = 16).
     const bool built = logDY == 7 || logDY == 8;
     const long items = S * (N / 64);
     if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);

@@ -379,7 +379,7 @@ int cu_count()
 }
 
 template <int LOGX, int LOGY>
-static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, long nimg, hipStream_t stream)
+static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, int nimg, hipStream_t stream)
 {
     using G = Geo2D<LOGX, LOGY>;
     static std::atomic<unsigned long long> served[2];
@@ -388,17 +388,17 @@ static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* ou
     if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse]); e != hipSuccess) return e;
     // persistent blocks: at most as many as fit at once (LDS allows one or two 1024-thread blocks per CU,
     // the thread count exactly one)
-    const long blocks = nimg < cu_count() ? nimg : cu_count();
+    const int blocks = nimg < cu_count() ? nimg : cu_count();
     if (inverse)
         hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, (int)nimg);
+                           out, nimg);
     else
         hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, (int)nimg);
+                           out, nimg);
     return hipGetLastError();
 }
 
-static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, const float2* in, float2* out, long nimg,
+static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, const float2* in, float2* out, int nimg,
                                         hipStream_t stream)
 {
     if (logDX == 8 && logDY == 8) return launch_image_kernel<8, 8>(inverse, in, out, nimg, stream);
@@ -408,12 +408,12 @@ static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, cons
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, long nimg, hipStream_t stream)
+hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, int nimg, hipStream_t stream)
 {
     return dispatch_image_kernel(false, logDX, logDY, x, spec, nimg, stream);
 }
 
-hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, long nimg, hipStream_t stream)
+hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, int nimg, hipStream_t stream)
 {
     return dispatch_image_kernel(true, logDX, logDY, spec, y, nimg, stream);
 }

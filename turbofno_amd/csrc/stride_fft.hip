@@ -128,7 +128,7 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
                   w3 = kTwiddle1024[(3 * t * (1024 / L)) & 1023];
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-            e[r] = cadd(cadd(lds[r * 16 + yl], cmulc(lds[(r + 16) * COLS + yl], w1)),
+            e[r] = cadd(cadd(lds[r * COLS + yl], cmulc(lds[(r + 16) * COLS + yl], w1)),
                         cadd(cmulc(lds[(r + 32) * COLS + yl], w2), cmulc(lds[(r + 48) * COLS + yl], w3)));
     } else {
 #pragma unroll

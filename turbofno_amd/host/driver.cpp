@@ -58,6 +58,8 @@ int main(int argc, char** argv)
     int algo = TURBOFNO_2D_AUTO;
     if (const char* e = getenv("TURBOFNO_2D_ALGO")) algo = atoi(e);
     if (const char* e = getenv("TURBOFNO_NTEST")) ntest = atoi(e) > 0 ? atoi(e) : ntest;
+    // measurement aid of these executables only (the library itself reads no environment): forces one of the fused 1D kernels
+    if (const char* e = getenv("TURBOFNO_1D_ALGO")) CHECK_TURBOFNO(turbofno_set_1d_algo(atoi(e)));
 
     for (const Problem& p : problems_from(argc, argv)) {
         // 1D: x[K][bs*dimX][DY]; 2D: x[K][bs][DX][DY]
