@@ -130,6 +130,21 @@ int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, co
                               float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
 
 /*
+ * The 2D layer for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. No counterpart in the reference (its mains allocate every buffer themselves,
+ * fused_trunc_2D.cu:68-85). Same arguments and results as turbofno_layer_2d, without the workspace: the
+ * intermediates live in a static device array of TURBOFNO_NOALLOC_SCRATCH_BYTES that every GPU the library runs on
+ * holds until the process ends. The call allocates and frees nothing. Problems whose intermediates
+ * (turbofno_layer_2d_workspace_bytes with the same arguments) exceed that size are refused with
+ * TURBOFNO_ERR_WORKSPACE; the headline problem bs=16, 256 x 256, K=N=64 fits exactly. The first call on a device
+ * resolves the array's address (make it outside any graph capture). All calls on one GPU share the one array:
+ * calls that overlap on the same GPU (different streams, different threads) race; calls on one stream are ordered.
+ */
+#define TURBOFNO_NOALLOC_SCRATCH_BYTES (64u << 20)
+int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,
+                              float alpha_re, float alpha_im, int algo, void* stream);
+
+/*
  * Process-wide choice of the fused 1D kernel behind turbofno_fused_fft_cgemm_ifft / turbofno_layer_1d and the Y stage
  * of the three-kernel 2D path (their reference-shaped signatures have no room for a selector): 0 = by problem size
  * (default), 1 = SIMT contraction, 2 / 3 = matrix cores with 512- / 256-thread blocks, 4 = matrix cores, 512 threads,

@@ -31,6 +31,10 @@ def test_layer_2d_rejects_mismatched_operands():
         tf.layer_2d(x, c64(64, 24))
     with pytest.raises(ValueError, match="y has shape"):
         tf.layer_2d(x, W, y=c64(64, 1, 128, 256))
+    with pytest.raises(ValueError, match="y has shape"):
+        tf.layer_2d_noalloc(x, W, c64(64, 2, 128, 128))
+    with pytest.raises(TypeError):
+        tf.layer_2d_noalloc(x, W, None)
     with pytest.raises(TypeError, match="on the GPU"):
         tf.layer_2d(x, W, y=c64(64, 1, 128, 128))
 
@@ -83,3 +87,10 @@ def test_1d_kernel_selector_round_trip():
         tf.set_1d_algo(7)
     assert tf.lib().turbofno_get_1d_algo() == 5           # a refused value changes nothing
     tf.set_1d_algo(prev)
+
+
+def test_noalloc_refuses_oversized_problem_without_gpu():
+    L = tf.lib()
+    # bs=32, 256 x 256, K=N=64: 128 MiB of intermediates, the static scratch holds 64 MiB; refused before any GPU call
+    rc = L.turbofno_layer_2d_noalloc(32, 256, 256, 64, 64, 1, 1, 1, 1.0, 0.0, 2, None)
+    assert rc == 3 and b"static scratch" in L.turbofno_last_error_string()

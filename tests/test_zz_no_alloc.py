@@ -1,0 +1,44 @@
+"""turbofno_layer_2d_noalloc (the 2D layer with its intermediates in the library's static device scratch) against
+turbofno_layer_2d on the same inputs: identical kernels on identical data, so the outputs must agree bit for bit; two
+calls in a row, the second with a smaller problem, so that whatever the first call left in the shared scratch is seen
+not to leak into the second. Also against the oracle, and the refusal of problems beyond the scratch size."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import turbofno_amd as tf
+from turbofno_amd import workloads
+from conftest import max_rel, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("algo", [2, 1, 0])
+def test_noalloc_matches_workspace_entry_point_twice(algo, tol):
+    shapes = [(4, 256, 256, 64, 64), (2, 128, 256, 24, 64)]           # second call: smaller in every dimension
+    if algo == 1:
+        shapes = [(1, 256, 256, 64, 64), (1, 128, 128, 16, 64)]       # three-kernel intermediates are 4x larger: stay within 64 MiB
+    for call, (bs, DX, DY, K, N) in enumerate(shapes):
+        print("noalloc call", call, "algo", algo, bs, DX, DY, K, N, flush=True)
+        x_h, W_h = workloads.uniform_2d(600 + call + algo, bs, DX, DY, K, N)
+        x, W = torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
+        y_ref = tf.layer_2d(x, W, alpha=1 - 1j, algo=algo)
+        y = torch.full((N, bs, DX, DY), complex(np.nan, np.nan), dtype=torch.complex64, device="cuda")
+        tf.layer_2d_noalloc(x, W, y, alpha=1 - 1j, algo=algo)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.float32), y_ref.view(torch.float32)), "outputs differ from turbofno_layer_2d"
+        ref = oracle.layer_2d(np.ascontiguousarray(x_h[:, :1]), W_h, 1 - 1j)
+        got = y[:, :1].cpu().numpy()
+        assert rel_l2(got, ref) <= tol["l2"] and max_rel(got, ref) <= tol["max"]
+
+
+def test_noalloc_refuses_problems_beyond_the_scratch():
+    x = torch.zeros((64, 1, 128, 128), dtype=torch.complex64, device="cuda")
+    W = torch.zeros((64, 64), dtype=torch.complex64, device="cuda")
+    y = torch.zeros((64, 1, 128, 128), dtype=torch.complex64, device="cuda")
+    L = tf.lib()
+    # claim bs = 32 at 256 x 256 (128 MiB of intermediates): refused on sizes alone, before any launch
+    rc = L.turbofno_layer_2d_noalloc(32, 256, 256, 64, 64, x.data_ptr(), W.data_ptr(), y.data_ptr(), 1.0, 0.0, 2, None)
+    assert rc == 3 and b"static scratch" in L.turbofno_last_error_string()
+    torch.cuda.synchronize()

@@ -20,6 +20,7 @@ from .api import (  # noqa: F401
     ifft_stride_DY,
     layer_1d,
     layer_2d,
+    layer_2d_noalloc,
     layer_2d_workspace_bytes,
     lib,
     library_path,

@@ -49,6 +49,7 @@ def lib():
         L.turbofno_ifft_stride_DY.argtypes = [i, vp, vp, i, l, vp]
         L.turbofno_fused_fft_cgemm.argtypes = [i, l, i, i, vp, vp, vp, f, f, f, f, vp]
         L.turbofno_fused_cgemm_ifft.argtypes = [i, l, i, i, vp, vp, vp, vp, f, f, f, f, vp]
+        L.turbofno_layer_2d_noalloc.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, i, vp]
         L.turbofno_set_1d_algo.argtypes = [i]
         L.turbofno_get_1d_algo.argtypes = []
         L.turbofno_get_1d_algo.restype = i
@@ -57,7 +58,7 @@ def lib():
         for name in ("turbofno_fused_fft_cgemm_ifft", "turbofno_fft_stride", "turbofno_ifft_stride",
                      "turbofno_layer_1d", "turbofno_layer_2d", "turbofno_fft2d_trunc", "turbofno_ifft2d_pad",
                      "turbofno_cgemm", "turbofno_fft_stride_DY", "turbofno_ifft_stride_DY", "turbofno_fused_fft_cgemm",
-                     "turbofno_fused_cgemm_ifft", "turbofno_set_1d_algo"):
+                     "turbofno_fused_cgemm_ifft", "turbofno_layer_2d_noalloc", "turbofno_set_1d_algo"):
             getattr(L, name).restype = i
         _LIB = L
     return _LIB
@@ -202,6 +203,18 @@ def layer_2d(x, W, y=None, alpha=1.0 + 0j, workspace=None, algo=0):
     a = complex(alpha)
     _check(lib().turbofno_layer_2d(bs, DX, DY, K, N, x.data_ptr(), W.data_ptr(), y.data_ptr(),
                                    a.real, a.imag, workspace.data_ptr(), workspace.numel(), algo, _stream()))
+    return y
+
+
+def layer_2d_noalloc(x, W, y, alpha=1.0 + 0j, algo=0):
+    """turbofno_layer_2d_noalloc: the 2D layer with its intermediates in the library's static device scratch.
+    `y` must be passed: nothing is allocated on this path."""
+    if y is None:
+        raise TypeError("y must be passed: this path allocates nothing")
+    K, bs, DX, DY, N, y = _layer_2d_operands(x, W, y)
+    a = complex(alpha)
+    _check(lib().turbofno_layer_2d_noalloc(bs, DX, DY, K, N, x.data_ptr(), W.data_ptr(), y.data_ptr(),
+                                           a.real, a.imag, algo, _stream()))
     return y
 
 

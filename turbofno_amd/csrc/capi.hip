@@ -264,4 +264,44 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
     return layer_2d_on(bs, DX, DY, K, N, x, W, y, alpha_re, alpha_im, workspace, workspace_bytes, "workspace", algo, stream);
 }
 
+// ---- the 2D layer for callers that cannot allocate -------------------------------------------------------------
+// The intermediates of the layer live in a file-scope device array instead of a caller-provided workspace. Every GPU
+// holds its own copy of the array at its own address (from module load until the process ends); that address is
+// resolved once per device, with that device current, and kept. Host code uses the resolved pointer only: the
+// array's name is a host-side stand-in, not a device address.
+static __device__ __align__(256) unsigned char scratch[TURBOFNO_NOALLOC_SCRATCH_BYTES];
+static std::atomic<void*> g_scratch_ptr[64];
+
+static int scratch_of_current_device(void** out)
+{
+    int dev = 0;
+    if (int rc = hip_status(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= 64) return fail(TURBOFNO_ERR_UNSUPPORTED, "device ordinal %d: the static scratch is tracked for ordinals below 64", dev);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (int rc = hip_status(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+        if (!p) return fail(TURBOFNO_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+        g_scratch_ptr[dev].store(p, std::memory_order_release);       // a racing thread resolves the same address
+    }
+    *out = p;
+    return TURBOFNO_OK;
+}
+
+int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,
+                              float alpha_re, float alpha_im, int algo, void* stream)
+{
+    // sizes first, so that an oversized problem is refused without touching the device
+    if (bs > 0 && DX > 0 && DY > 0 && K > 0 && N > 0) {
+        const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, algo);
+        if (need > (size_t)TURBOFNO_NOALLOC_SCRATCH_BYTES)
+            return fail(TURBOFNO_ERR_WORKSPACE,
+                        "the layer needs %zu bytes of intermediates, the static scratch holds %zu: use turbofno_layer_2d with "
+                        "a workspace, or split the batch", need, (size_t)TURBOFNO_NOALLOC_SCRATCH_BYTES);
+    }
+    void* ptr = nullptr;
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    return layer_2d_on(bs, DX, DY, K, N, x, W, y, alpha_re, alpha_im, ptr, (size_t)TURBOFNO_NOALLOC_SCRATCH_BYTES,
+                       "static scratch", algo, stream);
+}
+
 }  // extern "C"
