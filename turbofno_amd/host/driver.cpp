@@ -65,17 +65,14 @@ int main(int argc, char** argv)
         // 1D: x[K][bs*dimX][DY]; 2D: x[K][bs][DX][DY]
         const size_t per_channel = TURBOFNO_VARIANT_2D ? (size_t)p.bs * p.dx * p.dy : (size_t)p.bs * p.dx * p.dy;
         const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
-        float* hx = (float*)malloc(sizeof(float) * 2 * in_elems);
-        float* hw = (float*)malloc(sizeof(float) * 2 * w_elems);
         if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
-        generate_random_vector(hx, 2 * (long)in_elems);
-        generate_random_vector(hw, 2 * (long)w_elems);
+        const std::vector<float> hx = draw_random(2 * in_elems), hw = draw_random(2 * w_elems);
         void *dx = nullptr, *dw = nullptr, *dy = nullptr, *dws = nullptr;
         HIP_RT_CALL(hipMalloc(&dx, sizeof(float) * 2 * in_elems));
         HIP_RT_CALL(hipMalloc(&dw, sizeof(float) * 2 * w_elems));
         HIP_RT_CALL(hipMalloc(&dy, sizeof(float) * 2 * out_elems));
-        HIP_RT_CALL(hipMemcpy(dx, hx, sizeof(float) * 2 * in_elems, hipMemcpyHostToDevice));
-        HIP_RT_CALL(hipMemcpy(dw, hw, sizeof(float) * 2 * w_elems, hipMemcpyHostToDevice));
+        upload_tiled(dx, 2 * in_elems, hx);
+        upload_tiled(dw, 2 * w_elems, hw);
         size_t ws_bytes = 0;
         if (TURBOFNO_VARIANT_2D && TURBOFNO_VARIANT == 'D') {
             ws_bytes = turbofno_layer_2d_workspace_bytes(p.bs, p.dx, p.dy, p.k, p.n, algo);
@@ -159,7 +156,6 @@ int main(int argc, char** argv)
         if (dC) HIP_RT_CALL(hipFree(dC));
         if (t1) HIP_RT_CALL(hipFree(t1));
         if (t2) HIP_RT_CALL(hipFree(t2));
-        free(hx); free(hw);
     }
     return 0;
 }

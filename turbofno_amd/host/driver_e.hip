@@ -80,11 +80,8 @@ int main(int argc, char** argv)
         const long M = per_channel * keepx * 64;
         const size_t in_elems = (size_t)nin * DX * p.dy, out_elems = (size_t)nout * DX * p.dy;
         const size_t big = in_elems > out_elems ? in_elems : out_elems;
-        float* hx = (float*)malloc(sizeof(float) * 2 * in_elems);
-        float* hw = (float*)malloc(sizeof(float) * 2 * (size_t)p.k * p.n);
         if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
-        generate_random_vector(hx, 2 * (long)in_elems);
-        generate_random_vector(hw, 2L * p.k * p.n);
+        const std::vector<float> hx = draw_random(2 * in_elems), hw = draw_random(2 * (size_t)p.k * p.n);
         float2 *dx = nullptr, *dspec = nullptr, *dA = nullptr, *dW = nullptr, *dC = nullptr, *dy = nullptr;
         HIP_RT_CALL(hipMalloc(&dx, sizeof(float2) * in_elems));
         HIP_RT_CALL(hipMalloc(&dspec, sizeof(float2) * big));
@@ -92,8 +89,8 @@ int main(int argc, char** argv)
         HIP_RT_CALL(hipMalloc(&dA, sizeof(float2) * M * p.k));
         HIP_RT_CALL(hipMalloc(&dC, sizeof(float2) * M * p.n));
         HIP_RT_CALL(hipMalloc(&dW, sizeof(float2) * p.k * p.n));
-        HIP_RT_CALL(hipMemcpy(dx, hx, sizeof(float2) * in_elems, hipMemcpyHostToDevice));
-        HIP_RT_CALL(hipMemcpy(dW, hw, sizeof(float2) * p.k * p.n, hipMemcpyHostToDevice));
+        upload_tiled(dx, 2 * in_elems, hx);
+        upload_tiled(dW, 2 * (size_t)p.k * p.n, hw);
         HIP_RT_CALL(hipMemset(dC, 0, sizeof(float2) * M * p.n));
 
         hipfftHandle plan_in, plan_out;
@@ -148,7 +145,7 @@ int main(int argc, char** argv)
         HIP_RT_CALL(hipEventDestroy(t_begin)); HIP_RT_CALL(hipEventDestroy(t_end));
         HIP_RT_CALL(hipFree(dx)); HIP_RT_CALL(hipFree(dspec)); HIP_RT_CALL(hipFree(dy));
         HIP_RT_CALL(hipFree(dA)); HIP_RT_CALL(hipFree(dC)); HIP_RT_CALL(hipFree(dW));
-        free(hx); free(hw);
+
     }
     CHECK_BLAS(hipblasDestroy(blas));
     return 0;

@@ -38,6 +38,24 @@ void generate_random_vector(float* target, long n)
     }
 }
 
+std::vector<float> draw_random(size_t n)
+{
+    std::vector<float> h(n < ((size_t)1 << 22) ? n : ((size_t)1 << 22));
+    generate_random_vector(h.data(), (long)h.size());
+    return h;
+}
+
+void upload_tiled(void* device, size_t n, const std::vector<float>& values)
+{
+    const size_t drawn = values.size() < n ? values.size() : n;
+    HIP_RT_CALL(hipMemcpy(device, values.data(), sizeof(float) * drawn, hipMemcpyHostToDevice));
+    for (size_t filled = drawn; filled < n;) {               // doubling copies: the filled prefix onto what follows it
+        const size_t chunk = filled < n - filled ? filled : n - filled;
+        HIP_RT_CALL(hipMemcpy((float*)device + filled, device, sizeof(float) * chunk, hipMemcpyDeviceToDevice));
+        filled += chunk;
+    }
+}
+
 void print_output_digest(const void* device_y, size_t complex_elems)
 {
     std::vector<float> h(2 * complex_elems);

@@ -20,6 +20,16 @@ std::map<std::string, std::vector<int>> load_problem_config(const std::string& p
 // +-{0..9} * 1e-3 from rand(), unseeded: the reference's input distribution
 void generate_random_vector(float* target, long n);
 
+// Inputs of one problem in two steps, so that the draws from rand() can precede every HIP call of the problem (the HIP
+// runtime's own threads draw from rand() once it is initialised, which would make the values depend on timing):
+//   draw_random(n)          min(n, 2^22) values of generate_random_vector's distribution, exactly as the reference's mains
+//                           draw them (utils/utils.cu:37-43, fused.cu:61-62);
+//   upload_tiled(dev, n, v) fills a device buffer of n floats with v, repeated (device-to-device copies) when n is larger:
+//                           drawing gigabytes from rand() per problem takes longer than the whole sweep, and the reference
+//                           fills its one fixed-size buffer once per process instead (fused.cu:25-45,61).
+std::vector<float> draw_random(size_t n);
+void upload_tiled(void* device, size_t n, const std::vector<float>& values);
+
 // With TURBOFNO_DIGEST set in the environment the drivers print, after the warm-up launch of each problem, one
 // line "digest: <weighted sum re> <weighted sum im> <sum |y|^2>" of the output on stderr, and reseed rand() before
 // generating each problem's inputs: every variant of a problem then sees the same inputs and must print the same
