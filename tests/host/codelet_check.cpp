@@ -127,13 +127,29 @@ template <int LOGD> static double check_wide(bool backward)
             fwd_pass1(v, tw, g);
             for (int r = 0; r < 16; ++r) exch[t * 17 + r] = g[r];
         }
-        for (int m = 0; m < 64; ++m) {
-            const cpx X = wide_forward_mode<L>(exch.data(), m);
-            zd acc = 0;
-            for (int j = 0; j < D; ++j) acc += zd(x[j].x, x[j].y) * std::polar(1.0, -2.0 * M_PI * ((long)j * m % D) / D);
-            num += std::norm(acc - zd(X.x, X.y));
-            den += std::norm(acc);
+        // second pass as the kernels run it: every lane's pruned 16-point transform, the small swap, the outer sums
+        std::vector<cpx> swap(64 * (L / 16));
+        for (int l = 0; l < L; ++l) {
+            cpx inner[4];
+            wide_forward_inner<L>(exch.data(), 1, l, inner);
+            for (int c = 0; c < 4; ++c) swap[wide_swap_index<L>(l / (L / 16), c, l % (L / 16))] = inner[c];
         }
+        std::vector<int> seen(64, 0);
+        for (int l = 0; l < L; ++l) {
+            cpx out[64 / L];
+            wide_forward_outer<L>(swap.data(), 1, l, out);
+            for (int j = 0; j < 64 / L; ++j) {
+                const int m = wide_mode<L>(l, j);
+                seen[m]++;
+                const cpx X = out[j];
+                zd acc = 0;
+                for (int jj = 0; jj < D; ++jj) acc += zd(x[jj].x, x[jj].y) * std::polar(1.0, -2.0 * M_PI * ((long)jj * m % D) / D);
+                num += std::norm(acc - zd(X.x, X.y));
+                den += std::norm(acc);
+            }
+        }
+        for (int m = 0; m < 64; ++m)
+            if (seen[m] != 1) { printf("mode %d produced %d times\n", m, seen[m]); exit(1); }
     } else {
         for (int m = 0; m < 64; ++m) exch[m] = make_float2((float)frand(), (float)frand());
         std::vector<cpx> y(D);

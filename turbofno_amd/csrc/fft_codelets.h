@@ -310,20 +310,42 @@ TFNO_DEV void inv_pass2(cpx (&e)[16], const cpx (&tw)[16], cpx (&y)[16])
     for (int i = 0; i < 16; ++i) y[i] = e[fft16_slot(i)];
 }
 
-// Lengths 512 and 1024 (L = 32 or 64 lanes per signal). The second pass is no longer a 16- or 8-point transform
-// in registers: after the exchange a lane forms each retained mode as a direct L-term sum, and before the backward
-// exchange each lane builds its 16 first-pass inputs from all 64 modes. Both take their L-point twiddles from the
-// 1024-entry table. `exch` is the group's exchange region as the other lanes left it (pitch-17 rows of first-pass
-// results for the forward direction; the 64 modes in natural order for the backward direction).
-//
-// Forward: mode m = r + 16 c (r = m % 16, c = m / 16 < 4):  X[m] = sum_{tt<L} exch[tt*17 + r] * w_L^(tt c).
-template <int L> TFNO_DEV cpx wide_forward_mode(const cpx* exch, int m)
+// Lengths 512 and 1024 (L = 32 or 64 lanes per signal). After the exchange E[tt][r] (tt < L lanes, r < 16: first-pass
+// results, already twiddled) the retained modes are  X[r + 16 c] = sum_{tt<L} E[tt][r] w_L^(tt c),  c < 4.  Split
+// tt = a + A b with A = L/16 (2 or 4) and b < 16:
+//     inner_a[c]  = sum_b E[a + A b][r] w16^(b c)       a pruned 16-point transform (dft16_first4), one (a, r) per lane
+//     X[r + 16 c] = sum_{a<A} w_L^(a c) inner_a[c]      the A lanes of one r swap their inner values (a second, small
+//                                                       exchange of 4 values per lane) and each finishes 4 / A modes
+// i.e. 16 + 4 exchange reads and ~150 flops per lane instead of the L reads and L complex multiply-adds of a direct sum.
+// Second-pass lane l = A r + a  (r = l / A, a = l % A) ends up with modes wide_mode<L>(l, j), j < 4 / A.
+// `es` is the element stride of the exchange arrays (1 when a lane group has its own region; the number of columns
+// when a block transforms several columns side by side).
+template <int L> TFNO_DEV constexpr int wide_mode(int l, int j) { return (l / (L / 16)) + 16 * ((l % (L / 16)) * (64 / L) + j); }
+// where lane (a', r) parks inner_a'[c] for the lane that finishes c
+template <int L> TFNO_DEV constexpr int wide_swap_index(int r, int c, int a) { return (r * 4 + c) * (L / 16) + a; }
+
+template <int L> TFNO_DEV void wide_forward_inner(const cpx* exch, int es, int l, cpx (&inner)[4])
 {
-    const int r = m & 15, c = m >> 4;
-    cpx acc = make_float2(0.f, 0.f);
-#pragma unroll 8
-    for (int tt = 0; tt < L; ++tt) cfma(acc, exch[tt * 17 + r], kTwiddle1024[(tt * c * (1024 / L)) & 1023]);
-    return acc;
+    constexpr int A = L / 16;
+    const int r = l / A, a = l % A;
+    cpx u[16];
+#pragma unroll
+    for (int b = 0; b < 16; ++b) u[b] = exch[((a + A * b) * 17 + r) * es];
+    dft16_first4<-1>(u, inner);
+}
+template <int L> TFNO_DEV void wide_forward_outer(const cpx* swap, int es, int l, cpx (&out)[64 / L])
+{
+    constexpr int A = L / 16, MM = 64 / L;
+    const int r = l / A, a = l % A;
+#pragma unroll
+    for (int j = 0; j < MM; ++j) {
+        const int c = a * MM + j;
+        cpx acc = swap[wide_swap_index<L>(r, c, 0) * es];
+#pragma unroll
+        for (int ap = 1; ap < A; ++ap)
+            cfma(acc, swap[wide_swap_index<L>(r, c, ap) * es], kTwiddle1024[(ap * c * (1024 / L)) & 1023]);
+        out[j] = acc;
+    }
 }
 // Backward: first-pass input r of lane t:  e[r] = sum_{c<4} C[r + 16 c] * conj(w_L^(t c)), C = exch[0..63].
 template <int L> TFNO_DEV void wide_backward_inputs(const cpx* exch, int t, cpx (&e)[16])

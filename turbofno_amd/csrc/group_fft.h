@@ -19,8 +19,17 @@ template <int LOGDY> struct Geo1D {
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * SW_PITCH + GROUPS * EXCH);
 };
 
+// Mode that lane t of an L-lane group holds in out[mm] after a forward transform.
+template <int LOGDY> TFNO_DEV constexpr int forward_mode_of_lane(int t, int mm)
+{
+    constexpr int L = (1 << LOGDY) / 16;
+    if constexpr (L >= 32) return wide_mode<L>(t, mm);
+    else return t + L * mm;
+}
+
 // second half of the forward transform: exchange of the twiddled first-pass results g[] inside the
-// L-lane group, then the pruned L-point DFT. On return lane `t` holds modes m = t + L*mm in out[mm].
+// L-lane group, then the pruned L-point DFT. On return lane `t` holds mode forward_mode_of_lane<LOGDY>(t, mm) in
+// out[mm]: t + L*mm for lengths 128 and 256.
 template <int LOGDY>
 TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
 {
@@ -35,8 +44,15 @@ TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&o
         for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
         dft16_first4<-1>(u, out);                       // out[s] = X[t + 16 s]
     } else if constexpr (L >= 32) {
+        // lengths 512 / 1024: pruned second pass with a second small exchange; NOTE the lane-to-mode map of the result
+        // is wide_mode<L>(t, mm), not t + L*mm (forward_mode_of_lane below)
+        cpx inner[4];
+        wide_forward_inner<L>(exch, 1, t, inner);
+        wave_lds_fence();                                // every lane of the group has read the first exchange
 #pragma unroll
-        for (int mm = 0; mm < 64 / L; ++mm) out[mm] = wide_forward_mode<L>(exch, t + L * mm);
+        for (int c = 0; c < 4; ++c) exch[wide_swap_index<L>(t / (L / 16), c, t % (L / 16))] = inner[c];
+        wave_lds_fence();
+        wide_forward_outer<L>(exch, 1, t, out);
     } else {
         cpx u0[8], u1[8], o0[4], o1[4];
 #pragma unroll
@@ -49,7 +65,7 @@ TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&o
 }
 
 // forward transform of one signal by one L-lane group; lane t holds samples t + L*i in v[].
-// On return lane `t` holds modes m = t + L*mm in out[mm].
+// On return lane `t` holds mode forward_mode_of_lane<LOGDY>(t, mm) in out[mm].
 template <int LOGDY>
 TFNO_DEV void group_forward(cpx (&v)[16], const cpx (&tw)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
 {

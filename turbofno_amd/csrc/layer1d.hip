@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
                 for (int a = 0; a < MM; ++a) out[a] = make_float2(0.f, 0.f);
             }
 #pragma unroll
-            for (int a = 0; a < MM; ++a) sA[g * G::SA_PITCH + t + L * a] = out[a];
+            for (int a = 0; a < MM; ++a) sA[g * G::SA_PITCH + (PAIR ? t + L * a : forward_mode_of_lane<LOGDY>(t, a))] = out[a];
         } else {
             // A tile of the chunk: 64 contiguous rows (this block's signal) of GROUPS columns
 #pragma unroll
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
         __syncthreads();                                       // all exchanges done: sA may overwrite them
         if (g < kn) {
 #pragma unroll
-            for (int a = 0; a < MM; ++a) sA[g * PA + t + L * a] = out[a];
+            for (int a = 0; a < MM; ++a) sA[g * PA + (PAIR ? t + L * a : forward_mode_of_lane<LOGDY>(t, a))] = out[a];
         }
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
@@ -677,9 +677,9 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
 #pragma unroll
         for (int i = 0; i < 16; ++i) v[i] = src[L * i];
         group_forward<LOGDY>(v, tw, exch, t, o);
-        float2* dst = out + sig * 64 + t;
+        float2* dst = out + sig * 64;
 #pragma unroll
-        for (int a = 0; a < MM; ++a) dst[L * a] = o[a];
+        for (int a = 0; a < MM; ++a) dst[forward_mode_of_lane<LOGDY>(t, a)] = o[a];
     } else {
         const float2* src = in + sig * 64 + t;
         cpx c[MM], yv[16];
@@ -764,10 +764,12 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     //    it is ahead for every K from about four items per CU; at DY = 256, where the block kernels are closer to
     //    what the access pattern allows, from eight items per CU and not for 16 < K < 64;
     //  * in between, K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
-    //    its vector instructions there, up to half of which are the contraction;
+    //    its vector instructions there, up to half of which are the contraction (lengths 512 / 1024: a tie within a
+    //    few percent for every K, the SIMT kernel stays; on small grids the 512-thread kernel is 30-40 % ahead there too);
     //  * in between, K < 32: the SIMT kernel (three blocks per CU at DY = 256, two at DY = 128; no idle lanes in short
     //    chunks; a tie at K = 16).
-    const bool built = logDY == 7 || logDY == 8;
+    const bool built = logDY >= 7 && logDY <= 10;
+    const bool long_signal = logDY >= 9;            // 512 / 1024: on large grids the block kernels tie with the SIMT kernel
     const long items = S * (N / 64);
     if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
@@ -776,7 +778,7 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     if (algo == 0 && logDY == 8 && items >= 8L * cu_count() && (K <= 16 || K >= 64))
         return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     int pick = algo == 4 ? 2 : algo;
-    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 ? 3 : 1);
+    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 && !long_signal ? 3 : 1);
     // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
     // shares the spectra through LDS; level at K = 32)
     if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cu_count()))) {
@@ -798,6 +800,10 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream);
     if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream);
     if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 3 && logDY == 9) return launch_fused_mfma<9, 256>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 3 && logDY == 10) return launch_fused_mfma<10, 256>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 2 && logDY == 9) return launch_fused_mfma<9, 512>(S, N, K, x, W, y, alpha, stream);
+    if (pick == 2 && logDY == 10) return launch_fused_mfma<10, 512>(S, N, K, x, W, y, alpha, stream);
     return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream);
 }
 

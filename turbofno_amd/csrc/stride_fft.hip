@@ -45,17 +45,17 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void fft_stride_
     __syncthreads();
     float2* dst = out + sig * 64 * DY + y;
     if constexpr (L >= 32) {
-        // lengths 512 / 1024: each retained row m = t + L*mm is a direct L-term sum over the first-pass results
-        // (the same arithmetic as wide_forward_mode, on this kernel's [t][r][yl] exchange layout)
+        // lengths 512 / 1024: pruned second pass with a second, small exchange (wide_forward_inner / _outer on this
+        // kernel's [t][r][yl] layout); thread (yl, t) ends up with rows wide_mode<L>(t, mm)
+        cpx inner[4], o[64 / L];
+        wide_forward_inner<L>(lds + yl, COLS, t, inner);
+        __syncthreads();
 #pragma unroll
-        for (int mm = 0; mm < 64 / L; ++mm) {
-            const int m = t + L * mm, r = m & 15, c = m >> 4;
-            cpx acc = make_float2(0.f, 0.f);
-#pragma unroll 8
-            for (int tt = 0; tt < L; ++tt)
-                cfma(acc, lds[(tt * 17 + r) * COLS + yl], kTwiddle1024[(tt * c * (1024 / L)) & 1023]);
-            dst[(long)m * DY] = acc;
-        }
+        for (int c = 0; c < 4; ++c) lds[wide_swap_index<L>(t / (L / 16), c, t % (L / 16)) * COLS + yl] = inner[c];
+        __syncthreads();
+        wide_forward_outer<L>(lds + yl, COLS, t, o);
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) dst[(long)wide_mode<L>(t, mm) * DY] = o[mm];
     } else if constexpr (L == 16) {
         cpx u[16], o[4];
 #pragma unroll
