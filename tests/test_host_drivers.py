@@ -57,8 +57,28 @@ def test_driver_result_lines(tmp_path):
     assert got == [(1, 128, 128, 64, 8), (1, 128, 128, 64, 16), (1, 256, 128, 64, 8), (1, 256, 128, 64, 16)], lines
 
 
-def _run_variant(exe, args):
+def test_seeded_input_generators(tmp_path):
+    """the C++ generators of the benchmark configurations' inputs: ranges, unit variance, smoothness, reproducibility"""
+    exe = str(tmp_path / "inputs_check")
+    subprocess.run(["g++", "-O2", "-std=c++17", os.path.join(ROOT, "tests", "host", "inputs_check.cpp"),
+                    os.path.join(ROOT, "turbofno_amd", "host", "inputs.cpp"), "-o", exe], check=True)
+    rows = {ln.split()[0]: [float(v) for v in ln.split()[1:]] for ln in
+            subprocess.run([exe], check=True, capture_output=True, text=True).stdout.splitlines()}
+    mn, mx, mean, var, low = rows["uniform"]
+    assert -1.0 <= mn < -0.99 and 0.99 < mx <= 1.0 and abs(mean) < 0.02 and abs(var - 2.0 / 3.0) < 0.03 and low < 0.7
+    mn, mx, mean, var, low = rows["smooth"]
+    assert abs(var - 8.0) < 0.5 and low > 0.999                    # eight unit sinusoids per part, all below bin 33
+    mn, mx, mean, var, low = rows["vorticity"]
+    assert abs(var - 1.0) < 1e-4 and low > 0.99                    # unit variance per channel, red spectrum
+    assert rows["reproducible"] == [1.0] and rows["differs"] == [1.0]
+    wmax, wvar = rows["weights"]
+    assert wmax <= 0.25 + 1e-6 and abs(wvar - 2.0) < 0.2             # uniform / sqrt(16); K * var of complex normal / sqrt(K) = 2
+
+
+def _run_variant(exe, args, inputs=None):
     env = dict(os.environ, TURBOFNO_DIGEST="1", TURBOFNO_NTEST="2")
+    if inputs:
+        env["TURBOFNO_INPUTS"] = inputs
     r = subprocess.run([exe] + [str(a) for a in args], check=True, capture_output=True, text=True, timeout=100, env=env)
     digest = [float(v) for v in re.search(r"digest: (\S+) (\S+) (\S+)", r.stderr).groups()]
     return r.stdout, digest
@@ -89,3 +109,24 @@ def test_all_variants_agree(dim, args):
         scale = (ref[2] * nelem) ** 0.5          # bound of a weighted sum of nelem terms with that l2
         assert abs(dg[2] - ref[2]) <= 1e-4 * ref[2], (v, dg, ref)
         assert abs(dg[0] - ref[0]) <= 1e-5 * scale and abs(dg[1] - ref[1]) <= 1e-5 * scale, (v, dg, ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,args,inputs", [("1D", (8, 1, 256, 128, 64), "smooth"), ("2D", (2, 256, 256, 64, 16), "vorticity"),
+                                             ("2D", (1, 128, 128, 64, 16), "uniform")])
+def test_variants_agree_on_seeded_inputs(dim, args, inputs):
+    """TURBOFNO_INPUTS selects the seeded generators of the benchmark configurations: the fully fused (D) and the library
+    (E: hipFFT + hipBLAS) executables must agree on them as well"""
+    ref = None
+    for v in "DE":
+        exe = os.path.join(ROOT, "bin", f"TurboFNO_{dim}_{v}")
+        print(exe, args, inputs, flush=True)
+        out, dg = _run_variant(exe, args, inputs)
+        assert dg[2] > 0
+        if ref is None:
+            ref = dg
+            continue
+        nelem = args[0] * args[1] * args[2] * args[3]
+        scale = (ref[2] * nelem) ** 0.5
+        assert abs(dg[2] - ref[2]) <= 1e-4 * ref[2], (v, dg, ref)
+        assert abs(dg[0] - ref[0]) <= 2e-5 * scale and abs(dg[1] - ref[1]) <= 2e-5 * scale, (v, dg, ref)

@@ -19,6 +19,7 @@
 #include "../../include/turbofno.h"
 #include "TurboFNO.h"
 #include "utils.h"
+#include "inputs.h"
 #include <cmath>
 #include <cstring>
 #include <string>
@@ -66,7 +67,13 @@ int main(int argc, char** argv)
         const size_t per_channel = TURBOFNO_VARIANT_2D ? (size_t)p.bs * p.dx * p.dy : (size_t)p.bs * p.dx * p.dy;
         const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
         if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
-        const std::vector<float> hx = draw_random(2 * in_elems), hw = draw_random(2 * w_elems);
+        // inputs: the reference's rand() fill, or (TURBOFNO_INPUTS) one of the seeded distributions of the benchmark configurations
+        const InputKind kind = input_kind_from_name(getenv("TURBOFNO_INPUTS"));
+        const uint64_t seed = getenv("TURBOFNO_SEED") ? strtoull(getenv("TURBOFNO_SEED"), nullptr, 0) : default_seed(kind);
+        const bool seeded = kind != InputKind::reference_rand;
+        const long signals = TURBOFNO_VARIANT_2D ? (long)p.bs * p.dx : (long)p.bs * p.dx;
+        const std::vector<float> hx = seeded ? generate_inputs(kind, seed, p.k, signals, TURBOFNO_VARIANT_2D ? p.dx : 0, p.dy) : draw_random(2 * in_elems);
+        const std::vector<float> hw = seeded ? generate_weights(kind, seed, p.k, p.n) : draw_random(2 * w_elems);
         void *dx = nullptr, *dw = nullptr, *dy = nullptr, *dws = nullptr;
         HIP_RT_CALL(hipMalloc(&dx, sizeof(float) * 2 * in_elems));
         HIP_RT_CALL(hipMalloc(&dw, sizeof(float) * 2 * w_elems));

@@ -11,6 +11,7 @@
 // (2D_E.../fused_trunc_2D.cu:260); the label printed here is "2D_E".
 #include "TurboFNO.h"
 #include "utils.h"
+#include "inputs.h"
 #include <hipblas/hipblas.h>
 #include <hipfft/hipfft.h>
 #include <cmath>
@@ -81,7 +82,11 @@ int main(int argc, char** argv)
         const size_t in_elems = (size_t)nin * DX * p.dy, out_elems = (size_t)nout * DX * p.dy;
         const size_t big = in_elems > out_elems ? in_elems : out_elems;
         if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
-        const std::vector<float> hx = draw_random(2 * in_elems), hw = draw_random(2 * (size_t)p.k * p.n);
+        const InputKind kind = input_kind_from_name(getenv("TURBOFNO_INPUTS"));
+        const uint64_t seed = getenv("TURBOFNO_SEED") ? strtoull(getenv("TURBOFNO_SEED"), nullptr, 0) : default_seed(kind);
+        const bool seeded = kind != InputKind::reference_rand;
+        const std::vector<float> hx = seeded ? generate_inputs(kind, seed, p.k, per_channel * DX, TURBOFNO_VARIANT_2D ? p.dx : 0, p.dy) : draw_random(2 * in_elems);
+        const std::vector<float> hw = seeded ? generate_weights(kind, seed, p.k, p.n) : draw_random(2 * (size_t)p.k * p.n);
         float2 *dx = nullptr, *dspec = nullptr, *dA = nullptr, *dW = nullptr, *dC = nullptr, *dy = nullptr;
         HIP_RT_CALL(hipMalloc(&dx, sizeof(float2) * in_elems));
         HIP_RT_CALL(hipMalloc(&dspec, sizeof(float2) * big));
