@@ -63,6 +63,7 @@ int main(int argc, char** argv)
     if (const char* e = getenv("TURBOFNO_1D_ALGO")) CHECK_TURBOFNO(turbofno_set_1d_algo(atoi(e)));
 
     for (const Problem& p : problems_from(argc, argv)) {
+        if (p.k % THREADBLOCK_K != 0) { fprintf(stderr, "K=%d is not a multiple of %d: problem skipped\n", p.k, THREADBLOCK_K); continue; }
         // 1D: x[K][bs*dimX][DY]; 2D: x[K][bs][DX][DY]
         const size_t per_channel = TURBOFNO_VARIANT_2D ? (size_t)p.bs * p.dx * p.dy : (size_t)p.bs * p.dx * p.dy;
         const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
@@ -87,8 +88,8 @@ int main(int argc, char** argv)
         }
         // stage buffers of the unfused / half-fused variants: A[M x K], C[M x N] and, in 2D, the X-stage
         // intermediates t1[K*bs][64][DY], t2[N*bs][64][DY]
-        const long S = TURBOFNO_VARIANT_2D ? (long)p.bs * 64 : (long)p.bs * p.dx;   // signals per channel of the Y stage
-        const long M = 64 * S;
+        const long S = TURBOFNO_VARIANT_2D ? (long)p.bs * THREADBLOCK_M : (long)p.bs * p.dx;   // signals per channel of the Y stage
+        const long M = THREADBLOCK_M * S;
         const int logDY = (int)lround(log2((double)p.dy)), logDX = (int)lround(log2((double)p.dx));
         void *dA = nullptr, *dC = nullptr, *t1 = nullptr, *t2 = nullptr;
         if (TURBOFNO_VARIANT != 'D') {
@@ -112,7 +113,7 @@ int main(int argc, char** argv)
                 return;
             }
             if (TURBOFNO_VARIANT_2D) {
-                CHECK_TURBOFNO(turbofno_fft_stride(logDX, dx, t1, threadblock_bs, p.dy, (long)p.dy * p.k * p.bs, 64, nullptr));
+                CHECK_TURBOFNO(turbofno_fft_stride(logDX, dx, t1, threadblock_bs, p.dy, (long)p.dy * p.k * p.bs, THREADBLOCK_M, nullptr));
                 yin = t1; yout = t2;
             }
             if (TURBOFNO_VARIANT == 'A') {
@@ -127,7 +128,7 @@ int main(int argc, char** argv)
                 CHECK_TURBOFNO(turbofno_fused_cgemm_ifft(logDY, M, p.n, p.k, dA, dw, dC, yout, alpha_re, alpha_im, beta_re, beta_im, nullptr));
             }
             if (TURBOFNO_VARIANT_2D)
-                CHECK_TURBOFNO(turbofno_ifft_stride(logDX, t2, dy, threadblock_bs, p.dy, (long)p.dy * p.n * p.bs, 64, nullptr));
+                CHECK_TURBOFNO(turbofno_ifft_stride(logDX, t2, dy, threadblock_bs, p.dy, (long)p.dy * p.n * p.bs, THREADBLOCK_M, nullptr));
         };
         HIP_RT_CALL(hipDeviceSynchronize());
         launch();

@@ -75,10 +75,10 @@ int main(int argc, char** argv)
     for (const Problem& p : problems) {
         // 1D: nimg = bs*dimX signals per channel of length DY (DX plays no role: one row per signal)
         // 2D: nimg = bs images per channel of DX x DY
-        const int DX = TURBOFNO_VARIANT_2D ? p.dx : 1, keepx = TURBOFNO_VARIANT_2D ? 64 : 1;
+        const int DX = TURBOFNO_VARIANT_2D ? p.dx : 1, keepx = TURBOFNO_VARIANT_2D ? THREADBLOCK_M : 1;
         const long per_channel = TURBOFNO_VARIANT_2D ? (long)p.bs : (long)p.bs * p.dx;
         const long nin = per_channel * p.k, nout = per_channel * p.n;
-        const long M = per_channel * keepx * 64;
+        const long M = per_channel * keepx * THREADBLOCK_M;
         const size_t in_elems = (size_t)nin * DX * p.dy, out_elems = (size_t)nout * DX * p.dy;
         const size_t big = in_elems > out_elems ? in_elems : out_elems;
         if (getenv("TURBOFNO_DIGEST")) srand(1);   // same inputs in every executable, whatever the libraries drew from rand()
