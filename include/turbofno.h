@@ -152,7 +152,7 @@ int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* 
  * channels of an item split over the waves of a block. A value a kernel is not built for falls back to the choice by
  * size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
  */
-#define TURBOFNO_1D_ALGO_MAX 6
+#define TURBOFNO_1D_ALGO_MAX 7
 int turbofno_set_1d_algo(int algo);
 int turbofno_get_1d_algo(void);
 

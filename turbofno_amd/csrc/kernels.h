@@ -37,6 +37,14 @@ inline hipError_t allow_dynamic_lds(const void* kernel, size_t bytes, std::atomi
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream);
 
+// Cluster variant of the fused 1D layer (layer1d_cluster.hip): cluster size for a problem (0 = not applicable), the
+// launch (hipErrorNotReady when its exchange buffer cannot be provided), and the bound of its inter-block waits in
+// ticks of the 100 MHz wall clock.
+int cluster_size_1d(int logDY, long S, int N, int K);
+hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
+                                hipStream_t stream);
+void set_cluster_wait_ticks(unsigned long long ticks);
+
 // Halves of the fused kernel (variants B and C) and the stand-alone contiguous transforms (variant A).
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,
                                   float2 alpha, float2 beta, hipStream_t stream);

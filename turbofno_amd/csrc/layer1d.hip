@@ -753,7 +753,8 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
 
 // algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
 // 4 = as 2 with 32-channel output tiles, 5 = matrix cores, one wavefront per (signal set, output tile),
-// 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256)
+// 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256),
+// 7 = matrix cores, a cluster of blocks splits the K channels of one signal set (DY = 256, N = 64 / 128, small grids)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
@@ -777,6 +778,17 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
     if (algo == 0 && logDY == 8 && items >= 8L * cu_count() && (K <= 16 || K >= 64))
         return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
+    // small grids, 64 channels or more, N = 64 / 128: a cluster of blocks per signal set, no forward transform twice.
+    // Without its exchange buffer (first use inside a stream capture, out of memory) the kernels below take over.
+    if (algo == 7 || (algo == 0 && logDY == 8 && K >= 64)) {
+        const int P = cluster_size_1d(logDY, S, N, K);
+        if (P == 0 && algo == 7) return hipErrorInvalidValue;
+        if (P > 0) {
+            const hipError_t e = launch_fused_cluster(S, N, K, P, x, W, y, alpha, stream);
+            if (e != hipErrorNotReady) return e;
+            if (algo == 7) return e;
+        }
+    }
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 && !long_signal ? 3 : 1);
     // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that

@@ -1,0 +1,319 @@
+// Fused 1D spectral layer for SMALL grids with many channels (DY = 256): a CLUSTER of P workgroups shares one signal
+// set and splits its K input channels, so that no forward transform is computed twice.
+//
+// Same operands and result as fused_fft_cgemm_ifft_8 of the reference
+// (fusion_variants/1D_D_exp_fused_fft_cgemm_ifft/fused_fft_cgemm_ifft_7.cuh:9-222), whose (S, N/64) grid gives every
+// block of a signal set ALL K forward transforms. With few signal sets (S * N/64 well below the number of CUs) that
+// repetition is the critical path. Here member q of a cluster
+//   1. transforms channels [q K/P, (q+1) K/P) of the signal set (32 at a time, one per 16-lane group),
+//   2. multiplies them with the matching rows of W for ALL N output channels on v_mfma_f32_16x16x4_f32
+//      (spectra and the real-expanded W' tile staged through LDS as in fused_fft_mfma_ifft_kernel),
+//   3. publishes the partial products of the output channels it does not own to the other members through device
+//      memory, keeps its own N/P channels in LDS,
+//   4. waits (bounded) until all P members have published, adds the P-1 foreign partials to its own, runs the
+//      zero-padded backward transforms of its N/P channels and stores y.
+// Members of a cluster get block ids eight apart (same XCD, dispatched together). A waiting member only ever waits for
+// blocks with ids less than 8 P away, all of which the in-order dispatcher has started or will start without this
+// block's resources, whatever the grid size.
+//
+// Publication protocol: partials are written with device-scope stores (written through, complete when the wave's
+// store counter drains) and read with device-scope loads (never served from a stale private line), so no cache-wide
+// write-back or invalidate is needed: the producer waits for its stores, the block's first thread bumps the
+// cluster's arrival counter, consumers poll that counter. The counter is never reset: every launch adds exactly P,
+// launches that share a counter are ordered by their stream, so an arriving member that reads the old value v knows
+// the launch is complete at (v / P + 1) P. That also makes the kernel replayable from a captured graph.
+#include "group_fft.h"
+#include "kernels.h"
+
+#include <map>
+#include <mutex>
+
+namespace tfno {
+
+typedef float floatx4_cl __attribute__((ext_vector_type(4)));
+
+template <int NT> struct GeoCluster {
+    static constexpr int KC = 32;                               // channels per chunk = lane groups of a block
+    static constexpr int PA = 80, PC = 72;                      // pitches (complex) of the spectra tile and of the own product
+    static constexpr int EXCH = 16 * 17;
+    static constexpr int REGION0 = KC * EXCH;                   // exchange regions | spectra tile sA[KC][PA]
+    // W' tile as kWHalf / kWGroup of the block kernels, widened to 2 NT rows
+    static constexpr int WHALF = 8 * NT + 4, WGROUP = 2 * WHALF;
+    static constexpr int WTILE = (KC / 4) * WGROUP / 2;         // complex units
+    static constexpr int REGION1 = WTILE > 32 * PC ? WTILE : 32 * PC;   // W' tile | own product sC[<=32][PC]
+    static constexpr int NTW = NT / 16;                         // 16 x 16 tiles per wave: one m tile x NTW n' tiles
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
+    static_assert(KC * PA <= REGION0, "spectra tile must fit the exchange regions");
+};
+
+namespace {
+
+constexpr int kArriveStride = 32;                               // counters 128 bytes apart: one line per cluster
+
+__device__ __forceinline__ unsigned counter_load(const unsigned* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void stores_complete() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ cpx load_published(const cpx* p)
+{
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(cpx, v);
+}
+__device__ __forceinline__ void store_published(cpx* p, cpx v)
+{
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace
+
+// part[S][P][N][64]: partial products by (signal set, producing member); arrive[S * kArriveStride]; *gave_up (host
+// memory the device can write) is set when a wait ran into its bound, after which the output of that launch is invalid.
+template <int NT>
+__global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S, int K, int P, const float2* __restrict__ x,
+                                                                          const float2* __restrict__ W, float2* __restrict__ y,
+                                                                          float2 alpha, float2* part, unsigned* arrive,
+                                                                          unsigned* gave_up, unsigned long long wait_ticks)
+{
+    using G = GeoCluster<NT>;
+    constexpr int DY = 256, N = NT, KC = G::KC, PA = G::PA, PC = G::PC, NTW = G::NTW;
+    extern __shared__ float2 lds[];
+    float2* sA = lds;
+    float* sW = reinterpret_cast<float*>(lds + G::REGION0);
+    float2* sC = lds + G::REGION0;
+
+    const int tid = threadIdx.x;
+    const int g = tid >> 4, t = tid & 15;                       // transform role: lane group g, lane t
+    const int wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;   // matrix role
+    const int mt = wave & 3, nt0 = (wave >> 2) * NTW;
+    // block id -> (signal set, member): ids of one cluster are eight apart
+    const unsigned id = blockIdx.x, j = id >> 3;
+    const int q = (int)(j % (unsigned)P);
+    const long s = (long)(j / (unsigned)P) * 8 + (id & 7);
+    if (s >= S) return;                                         // padding of the last group of eight clusters
+    const int KB = K / P, NB = N / P, kbase = q * KB;
+    float2* exch = lds + g * G::EXCH;
+
+    cpx tw[16];
+    load_lane_twiddles<8>(t, tw);
+    floatx4_cl acc[NTW];
+#pragma unroll
+    for (int i = 0; i < NTW; ++i) acc[i] = floatx4_cl{ 0.f, 0.f, 0.f, 0.f };
+
+    const float2* src = x + ((long)(kbase + g) * S + s) * DY + t;
+    auto issue = [&](cpx (&dst)[16], int kc) {
+        const float2* p = src + (long)kc * S * DY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[i] = p[16 * i];
+    };
+    cpx v[16];
+    if (g < KB) issue(v, 0);
+
+    for (int kc = 0; kc < KB; kc += KC) {
+        const int kn = (KB - kc) < KC ? (KB - kc) : KC;         // multiple of 4
+        constexpr int WPT = KC * NT / 512;
+        float2 wv[WPT];
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * 512;
+            const int k = idx % KC, n = idx / KC;
+            wv[u] = (k < kn) ? W[(kbase + kc + k) + (long)n * K] : make_float2(0.f, 0.f);
+        }
+        cpx out[4];
+        if (g < kn) {
+            cpx gg[16];
+            fwd_pass1(v, tw, gg);
+            if (kc + KC + g < KB) issue(v, kc + KC);
+            group_forward_finish<8>(gg, exch, t, out);
+        }
+        __syncthreads();                                        // all exchanges done: sA may overwrite them
+        if (g < kn) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) sA[g * PA + t + 16 * a] = out[a];
+        }
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * 512;
+            const int k = idx % KC, n = idx / KC;
+            const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
+            float* dstw = &sW[(k >> 2) * G::WGROUP + ((k & 3) >> 1) * G::WHALF + (2 * n) * 4 + (k & 1) * 2];
+            *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
+            *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
+        }
+        __syncthreads();
+        const float2* arow = sA + kq * PA + mt * 16 + col;
+        const float* wrow = sW + (kq >> 1) * G::WHALF + (nt0 * 16 + col) * 4 + (kq & 1) * 2;
+        for (int kg = 0; kg < kn / 4; ++kg) {
+            const float2 b = arow[kg * 4 * PA];
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) {
+                const float2 a = *reinterpret_cast<const float2*>(wrow + kg * G::WGROUP + i * 64);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[i], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                        // sA / sW are free again (next chunk, or sC below)
+    }
+
+    // D[row = 4 kq + v][col] of tile i: output channel n = 8 (nt0 + i) + 2 kq + (v >> 1), re | im = v & 1, mode 16 mt + col.
+    // NB is a multiple of 8, so the owner n / NB is the same for the whole tile.
+    {
+        float2* mine = part + ((long)(s * P + q) * N) * 64 + mt * 16 + col;
+#pragma unroll
+        for (int i = 0; i < NTW; ++i) {
+            const int n = 8 * (nt0 + i) + 2 * kq;
+            const float2 c0 = make_float2(acc[i][0], acc[i][1]), c1 = make_float2(acc[i][2], acc[i][3]);
+            if (n / NB == q) {
+                sC[(n - NB * q) * PC + mt * 16 + col] = c0;
+                sC[(n + 1 - NB * q) * PC + mt * 16 + col] = c1;
+            } else {
+                store_published(mine + (long)n * 64, c0);
+                store_published(mine + (long)(n + 1) * 64, c1);
+            }
+        }
+    }
+    stores_complete();
+    __syncthreads();
+    if (tid == 0) {
+        unsigned* ctr = arrive + s * kArriveStride;
+        const unsigned old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned target = (old / (unsigned)P + 1u) * (unsigned)P;     // P is a power of two: consistent under wrap-around
+        if ((int)(counter_load(ctr) - target) < 0) {
+            const unsigned long long t0 = wall_clock64();
+            while ((int)(counter_load(ctr) - target) < 0) {
+                if (wall_clock64() - t0 > wait_ticks) {
+                    __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+        }
+    }
+    __syncthreads();
+    asm volatile("" ::: "memory");                              // the loads below are issued after the counter was seen
+
+    if (g < NB) {
+        const int n = NB * q + g;
+        cpx c[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) c[a] = sC[g * PC + t + 16 * a];
+        for (int qq = 1; qq < P; ++qq) {
+            const int from = (q + qq) & (P - 1);
+            const float2* p = part + ((long)(s * P + from) * N + n) * 64 + t;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], load_published(p + 16 * a));
+        }
+        cpx yv[16];
+        group_backward<8>(c, tw, exch, t, yv);
+        float2* dst = y + ((long)n * S + s) * DY + t;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, yv[i]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Exchange memory: one buffer per (device, stream) that has used this path, grown on demand and kept until the process
+// ends. Calls on one stream are ordered and may share it; calls on different streams get different buffers.
+namespace {
+
+struct Exchange {
+    float2* part = nullptr;
+    size_t part_bytes = 0;
+    unsigned* arrive = nullptr;
+    long clusters = 0;
+    unsigned* gave_up = nullptr;    // pinned host word, written by a kernel whose wait ran into its bound
+};
+
+std::mutex g_exchange_mutex;
+std::map<std::pair<int, hipStream_t>, Exchange> g_exchange;
+std::atomic<unsigned long long> g_wait_ticks{ 200000000ull };    // 2 s of the 100 MHz wall clock
+
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return st != hipStreamCaptureStatusNone;
+}
+
+// Returns the buffer of (current device, stream), sized for `clusters` signal sets of `bytes_per_cluster`; nullptr when
+// it cannot be provided (allocation failed, or it would have to be allocated while the stream is being captured).
+Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_cluster)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_exchange_mutex);
+    Exchange& e = g_exchange[{ dev, stream }];
+    const size_t need = (size_t)clusters * bytes_per_cluster;
+    if (e.part_bytes >= need && e.clusters >= clusters && e.gave_up) return &e;
+    if (stream_is_capturing(stream)) return nullptr;
+    if (!e.gave_up) {
+        if (hipHostMalloc(reinterpret_cast<void**>(&e.gave_up), 64, hipHostMallocDefault) != hipSuccess) { e.gave_up = nullptr; return nullptr; }
+        *e.gave_up = 0;
+    }
+    if (e.part_bytes < need) {
+        if (e.part) (void)hipFree(e.part);                      // hipFree waits for the work that may still use it
+        e.part = nullptr;
+        e.part_bytes = 0;
+        if (hipMalloc(reinterpret_cast<void**>(&e.part), need) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        e.part_bytes = need;
+    }
+    if (e.clusters < clusters) {
+        if (e.arrive) (void)hipFree(e.arrive);
+        e.arrive = nullptr;
+        e.clusters = 0;
+        const size_t bytes = sizeof(unsigned) * kArriveStride * (size_t)clusters;
+        if (hipMalloc(reinterpret_cast<void**>(&e.arrive), bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        if (hipMemset(e.arrive, 0, bytes) != hipSuccess) return nullptr;      // synchronous, once per growth
+        e.clusters = clusters;
+    }
+    return &e;
+}
+
+template <int NT>
+hipError_t launch_cluster_t(long S, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha, Exchange* e,
+                            hipStream_t stream)
+{
+    using G = GeoCluster<NT>;
+    static std::atomic<unsigned long long> served;
+    if (hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_cluster_kernel<NT>), G::LDS_BYTES, served);
+        err != hipSuccess)
+        return err;
+    const long blocks = ((S + 7) / 8) * 8 * P;
+    hipLaunchKernelGGL(fused_fft_mfma_ifft_cluster_kernel<NT>, dim3((unsigned)blocks), dim3(512), G::LDS_BYTES, stream, (int)S, K, P,
+                       x, W, y, alpha, e->part, e->arrive, e->gave_up, g_wait_ticks.load(std::memory_order_relaxed));
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// Cluster size for (S, N, K), or 0 when this kernel does not apply: N in {64, 128}, every member gets a multiple of four
+// input channels and 8 ... 32 output channels, and the whole grid is resident at once (one block per CU).
+int cluster_size_1d(int logDY, long S, int N, int K)
+{
+    if (logDY != 8 || (N != 64 && N != 128) || S <= 0) return 0;
+    const long cus = cu_count();
+    int P = N / 32;
+    while (P < 8 && ((S + 7) / 8) * 8 * (2 * P) <= cus) P *= 2;
+    if (((S + 7) / 8) * 8 * P > cus) return 0;
+    if (K % (4 * P) != 0 || N / P < 8) return 0;
+    return P;
+}
+
+// hipErrorNotReady: the exchange buffer could not be provided (the caller falls back on a kernel without one);
+// hipErrorLaunchFailure: an earlier launch on this stream gave up waiting for a cluster member.
+hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
+                                hipStream_t stream)
+{
+    if (P < 2 || (P & (P - 1)) || K % (4 * P) || N % P || N / P > 32 || N / P < 8) return hipErrorInvalidValue;
+    Exchange* e = exchange_for(stream, S, sizeof(float2) * 64 * (size_t)N * P);
+    if (!e) return hipErrorNotReady;
+    if (*static_cast<volatile unsigned*>(e->gave_up)) {          // reported once; the arrival counters stay consistent
+        *e->gave_up = 0;
+        return hipErrorLaunchFailure;
+    }
+    if (N == 128) return launch_cluster_t<128>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 64) return launch_cluster_t<64>(S, K, P, x, W, y, alpha, e, stream);
+    return hipErrorInvalidValue;
+}
+
+void set_cluster_wait_ticks(unsigned long long ticks) { g_wait_ticks.store(ticks, std::memory_order_relaxed); }
+
+}  // namespace tfno
