@@ -33,6 +33,7 @@ extern "C" {
 #define TURBOFNO_ERR_UNSUPPORTED  2  /* transform length outside the built set                           */
 #define TURBOFNO_ERR_WORKSPACE    3  /* workspace missing or too small                                   */
 #define TURBOFNO_ERR_HIP          4  /* the HIP runtime reported a launch error                          */
+#define TURBOFNO_ERR_EXCHANGE     5  /* an earlier clustered launch on this stream gave up an inter-block wait */
 
 #define TURBOFNO_MODES 64
 
@@ -149,12 +150,29 @@ int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* 
  * of the three-kernel 2D path (their reference-shaped signatures have no room for a selector): 0 = by problem size
  * (default), 1 = SIMT contraction, 2 / 3 = matrix cores with 512- / 256-thread blocks, 4 = matrix cores, 512 threads,
  * 32-channel output tiles, 5 = matrix cores, one wavefront per signal set and output tile, 6 = matrix cores, the K
- * channels of an item split over the waves of a block. A value a kernel is not built for falls back to the choice by
- * size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
+ * channels of an item split over the waves of a block, 7 = matrix cores, the K channels of a signal set split over a
+ * cluster of blocks (see below). A value a kernel is not built for falls back to the choice by size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
  */
 #define TURBOFNO_1D_ALGO_MAX 7
 int turbofno_set_1d_algo(int algo);
 int turbofno_get_1d_algo(void);
+
+/*
+ * Clustered launches (no counterpart in the reference). On small grids with K >= 64 (DY = 256, N = 64 or 128, every
+ * block on a CU of its own) the fused 1D layer splits the K channels of a signal set over 2 - 8 blocks, which exchange
+ * partial products through a device buffer that the library owns: one per (device, stream) that has used this path,
+ * at most 512 N bytes per compute unit (16 MiB for N = 128 on 256 CUs), allocated on first use and kept until the
+ * process ends. Consequences for callers:
+ *   - calls on one stream are ordered and share the buffer; calls on different streams use different buffers;
+ *   - the first such call on a stream allocates (and synchronises the device once); inside a stream capture that is
+ *     not possible, and a kernel without the exchange runs instead. A captured launch keeps using the buffer of the
+ *     stream it was captured on: do not replay it concurrently with other 1D layer calls on that stream;
+ *   - every inter-block wait is bounded (default 2 s). A block that runs into the bound gives up, the launch completes
+ *     with invalid output, and the NEXT 1D layer call on that stream returns TURBOFNO_ERR_EXCHANGE once, without
+ *     launching. turbofno_set_exchange_wait_us changes the bound (microseconds, process-wide; 0 = give up at once,
+ *     for tests of this error path).
+ */
+int turbofno_set_exchange_wait_us(unsigned long long microseconds);
 
 /* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
 const char* turbofno_last_error_string(void);

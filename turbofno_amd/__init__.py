@@ -25,6 +25,7 @@ from .api import (  # noqa: F401
     lib,
     library_path,
     set_1d_algo,
+    set_exchange_wait_us,
 )
 
 ALGO_AUTO, ALGO_THREE_KERNEL, ALGO_WHOLE_IMAGE = 0, 1, 2

@@ -52,6 +52,8 @@ def lib():
         L.turbofno_layer_2d_noalloc.argtypes = [i, i, i, i, i, vp, vp, vp, f, f, i, vp]
         L.turbofno_set_1d_algo.argtypes = [i]
         L.turbofno_get_1d_algo.argtypes = []
+        L.turbofno_set_exchange_wait_us.argtypes = [ctypes.c_ulonglong]
+        L.turbofno_set_exchange_wait_us.restype = i
         L.turbofno_get_1d_algo.restype = i
         L.turbofno_last_error_string.restype = ctypes.c_char_p
         L.turbofno_abi_version.restype = i
@@ -108,6 +110,11 @@ def set_1d_algo(algo):
     prev = lib().turbofno_get_1d_algo()
     _check(lib().turbofno_set_1d_algo(int(algo)))
     return prev
+
+
+def set_exchange_wait_us(microseconds):
+    """Bound of the inter-block waits of the clustered 1D kernel (include/turbofno.h); 0 = give up at once."""
+    _check(lib().turbofno_set_exchange_wait_us(int(microseconds)))
 
 
 def fused_fft_cgemm_ifft(M, N, K, x, W, y, alpha=1.0 + 0j, beta=0j, C=None):

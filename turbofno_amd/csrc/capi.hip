@@ -22,6 +22,9 @@ int fail(int code, const char* fmt, ...)
 int hip_status(hipError_t e, const char* what)
 {
     if (e == hipSuccess) return TURBOFNO_OK;
+    if (e == hipErrorLaunchTimeOut)         // reported by the clustered 1D launcher, never by a launch itself
+        return fail(TURBOFNO_ERR_EXCHANGE, "%s: a block of an earlier clustered launch on this stream gave up waiting for its cluster; "
+                                           "that launch's output is invalid", what);
     return fail(TURBOFNO_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
@@ -72,7 +75,7 @@ const char* turbofno_last_error_string(void) { return g_err; }
 // the process-wide selector set by turbofno_set_1d_algo (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with
 // 512- / 256-thread blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one
 // wavefront per signal set and output tile, 6 matrix cores with the K channels of an item split over the waves of a
-// block) overrides the choice by size.
+// block, 7 matrix cores with the K channels of a signal set split over a cluster of blocks) overrides the choice by size.
 static std::atomic<int> g_algo_1d{ 0 };
 static int algo_1d() { return g_algo_1d.load(std::memory_order_relaxed); }
 
@@ -84,6 +87,12 @@ int turbofno_set_1d_algo(int algo)
 }
 
 int turbofno_get_1d_algo(void) { return algo_1d(); }
+
+int turbofno_set_exchange_wait_us(unsigned long long microseconds)
+{
+    tfno::set_cluster_wait_ticks(microseconds > (~0ull) / 100 ? ~0ull : microseconds * 100);   // 100 MHz wall clock
+    return TURBOFNO_OK;
+}
 
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream)

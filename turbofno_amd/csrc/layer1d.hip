@@ -782,12 +782,11 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     // Without its exchange buffer (first use inside a stream capture, out of memory) the kernels below take over.
     if (algo == 7 || (algo == 0 && logDY == 8 && K >= 64)) {
         const int P = cluster_size_1d(logDY, S, N, K);
-        if (P == 0 && algo == 7) return hipErrorInvalidValue;
         if (P > 0) {
             const hipError_t e = launch_fused_cluster(S, N, K, P, x, W, y, alpha, stream);
             if (e != hipErrorNotReady) return e;
-            if (algo == 7) return e;
         }
+        if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
     }
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 && !long_signal ? 3 : 1);

@@ -19,9 +19,9 @@
 // Publication protocol: partials are written with device-scope stores (written through, complete when the wave's
 // store counter drains) and read with device-scope loads (never served from a stale private line), so no cache-wide
 // write-back or invalidate is needed: the producer waits for its stores, the block's first thread bumps the
-// cluster's arrival counter, consumers poll that counter. The counter is never reset: every launch adds exactly P,
-// launches that share a counter are ordered by their stream, so an arriving member that reads the old value v knows
-// the launch is complete at (v / P + 1) P. That also makes the kernel replayable from a captured graph.
+// cluster's arrival counter, consumers poll that counter. The counter is never reset: every launch adds exactly 8
+// (8 / P per member), launches that share a counter are ordered by their stream, so an arriving member that reads the
+// old value v knows the launch is complete at (v / 8 + 1) 8. That also makes the kernel replayable from a captured graph.
 #include "group_fft.h"
 #include "kernels.h"
 
@@ -32,18 +32,22 @@ namespace tfno {
 
 typedef float floatx4_cl __attribute__((ext_vector_type(4)));
 
-template <int NT> struct GeoCluster {
-    static constexpr int KC = 32;                               // channels per chunk = lane groups of a block
+// NT = output channels of the layer, KC_ = channels per chunk (8, 16 or 32: lane groups that transform at a time)
+template <int NT, int KC_> struct GeoCluster {
+    static constexpr int KC = KC_;
     static constexpr int PA = 80, PC = 72;                      // pitches (complex) of the spectra tile and of the own product
     static constexpr int EXCH = 16 * 17;
-    static constexpr int REGION0 = KC * EXCH;                   // exchange regions | spectra tile sA[KC][PA]
-    // W' tile as kWHalf / kWGroup of the block kernels, widened to 2 NT rows
-    static constexpr int WHALF = 8 * NT + 4, WGROUP = 2 * WHALF;
-    static constexpr int WTILE = (KC / 4) * WGROUP / 2;         // complex units
-    static constexpr int REGION1 = WTILE > 32 * PC ? WTILE : 32 * PC;   // W' tile | own product sC[<=32][PC]
-    static constexpr int NTW = NT / 16;                         // 16 x 16 tiles per wave: one m tile x NTW n' tiles
-    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1);
+    static constexpr int REGION0 = 32 * EXCH;                   // exchange regions (32 for the backward pass) | spectra tile sA[KC][PA]
+    // W'' tile: three planes (c, d - c, c + d; alpha W = c + i d) of floats at (k / 4) * WGROUP + (k % 4) * WROW + n.
+    // An operand fetch (4 k x 16 n) reads 16 consecutive floats of four rows that are 16 banks apart; the group stride
+    // of 1 (mod 64 banks) spreads the tile build, whose lanes run along k, over the banks as well.
+    static constexpr int WROW = NT + 16, WGROUP = 4 * WROW + 1, WPLANE = (KC / 4) * WGROUP;
+    static constexpr int REGION1 = (3 * WPLANE + 1) / 2;        // complex units
+    static constexpr int REGION2 = 32 * PC;                     // own product sC[<= 32][PC]
+    static constexpr int TPW = NT / 32;                         // 16 n x 16 m tiles per wave (one m tile, TPW n tiles)
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1 + REGION2);
     static_assert(KC * PA <= REGION0, "spectra tile must fit the exchange regions");
+    static_assert(WROW % 64 == 16, "rows of an operand fetch must be 16 banks apart");
 };
 
 namespace {
@@ -67,23 +71,23 @@ __device__ __forceinline__ void store_published(cpx* p, cpx v)
 
 // part[S][P][N][64]: partial products by (signal set, producing member); arrive[S * kArriveStride]; *gave_up (host
 // memory the device can write) is set when a wait ran into its bound, after which the output of that launch is invalid.
-template <int NT>
+template <int NT, int KC_>
 __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S, int K, int P, const float2* __restrict__ x,
                                                                           const float2* __restrict__ W, float2* __restrict__ y,
                                                                           float2 alpha, float2* part, unsigned* arrive,
                                                                           unsigned* gave_up, unsigned long long wait_ticks)
 {
-    using G = GeoCluster<NT>;
-    constexpr int DY = 256, N = NT, KC = G::KC, PA = G::PA, PC = G::PC, NTW = G::NTW;
+    using G = GeoCluster<NT, KC_>;
+    constexpr int DY = 256, N = NT, KC = G::KC, PA = G::PA, PC = G::PC, TPW = G::TPW;
     extern __shared__ float2 lds[];
     float2* sA = lds;
     float* sW = reinterpret_cast<float*>(lds + G::REGION0);
-    float2* sC = lds + G::REGION0;
+    float2* sC = lds + G::REGION0 + G::REGION1;
 
     const int tid = threadIdx.x;
     const int g = tid >> 4, t = tid & 15;                       // transform role: lane group g, lane t
     const int wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;   // matrix role
-    const int mt = wave & 3, nt0 = (wave >> 2) * NTW;
+    const int mt = wave & 3, tile0 = (wave >> 2) * TPW;         // m tile, first of the wave's TPW n tiles
     // block id -> (signal set, member): ids of one cluster are eight apart
     const unsigned id = blockIdx.x, j = id >> 3;
     const int q = (int)(j % (unsigned)P);
@@ -91,12 +95,16 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
     if (s >= S) return;                                         // padding of the last group of eight clusters
     const int KB = K / P, NB = N / P, kbase = q * KB;
     float2* exch = lds + g * G::EXCH;
+    // The wave walks its n tiles in a rotated order that ends with the tiles this member owns: the partials of the
+    // other members' channels are then on their way while the matrix cores still work on the rest.
+    const int own_last = (q * NB + NB - 1) / 16;                // last tile with channels of this member
+    const int rot = (own_last >= tile0 && own_last < tile0 + TPW) ? ((own_last - tile0 + 1) & (TPW - 1)) : 0;
 
     cpx tw[16];
     load_lane_twiddles<8>(t, tw);
-    floatx4_cl acc[NTW];
+    floatx4_cl p1[TPW], p2[TPW], p3[TPW];
 #pragma unroll
-    for (int i = 0; i < NTW; ++i) acc[i] = floatx4_cl{ 0.f, 0.f, 0.f, 0.f };
+    for (int i = 0; i < TPW; ++i) p1[i] = p2[i] = p3[i] = floatx4_cl{ 0.f, 0.f, 0.f, 0.f };
 
     const float2* src = x + ((long)(kbase + g) * S + s) * DY + t;
     auto issue = [&](cpx (&dst)[16], int kc) {
@@ -105,77 +113,81 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
         for (int i = 0; i < 16; ++i) dst[i] = p[16 * i];
     };
     cpx v[16];
-    if (g < KB) issue(v, 0);
+    if (g < KC) issue(v, 0);
+    float2* mine = part + ((long)(s * P + q) * N) * 64 + mt * 16 + col;
 
     for (int kc = 0; kc < KB; kc += KC) {
-        const int kn = (KB - kc) < KC ? (KB - kc) : KC;         // multiple of 4
-        constexpr int WPT = KC * NT / 512;
+        const bool last = kc + KC >= KB;
+        // W chunk: lanes run along k, the contiguous direction of W[k + n*K]; the two halves of a wavefront take
+        // channels eight apart (eight banks apart in the tile)
+        constexpr int WPT = KC * NT / 512;                      // KB is a multiple of KC: every chunk is full
         float2 wv[WPT];
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * 512;
-            const int k = idx % KC, n = idx / KC;
-            wv[u] = (k < kn) ? W[(kbase + kc + k) + (long)n * K] : make_float2(0.f, 0.f);
+            const int k = idx % KC, r = idx / KC, n = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
+            wv[u] = W[(kbase + kc + k) + (long)n * K];
         }
         cpx out[4];
-        if (g < kn) {
+        if (g < KC) {
             cpx gg[16];
             fwd_pass1(v, tw, gg);
-            if (kc + KC + g < KB) issue(v, kc + KC);
+            if (kc + KC < KB) issue(v, kc + KC);
             group_forward_finish<8>(gg, exch, t, out);
         }
-        __syncthreads();                                        // all exchanges done: sA may overwrite them
-        if (g < kn) {
-#pragma unroll
-            for (int a = 0; a < 4; ++a) sA[g * PA + t + 16 * a] = out[a];
-        }
+        // W'' tile (its region is not shared with the transforms): built by whichever waves are done transforming
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * 512;
-            const int k = idx % KC, n = idx / KC;
-            const float2 w = make_float2(wv[u].x * alpha.x - wv[u].y * alpha.y, wv[u].x * alpha.y + wv[u].y * alpha.x);
-            float* dstw = &sW[(k >> 2) * G::WGROUP + ((k & 3) >> 1) * G::WHALF + (2 * n) * 4 + (k & 1) * 2];
-            *reinterpret_cast<float2*>(dstw) = make_float2(w.x, -w.y);
-            *reinterpret_cast<float2*>(dstw + 4) = make_float2(w.y, w.x);
+            const int k = idx % KC, r = idx / KC, n = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
+            const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+            float* dstw = &sW[(k >> 2) * G::WGROUP + (k & 3) * G::WROW + n];
+            dstw[0] = c;
+            dstw[G::WPLANE] = d - c;
+            dstw[2 * G::WPLANE] = c + d;
+        }
+        __syncthreads();                                        // all exchanges done: sA may overwrite them
+        if (g < KC) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) sA[g * PA + t + 16 * a] = out[a];
         }
         __syncthreads();
         const float2* arow = sA + kq * PA + mt * 16 + col;
-        const float* wrow = sW + (kq >> 1) * G::WHALF + (nt0 * 16 + col) * 4 + (kq & 1) * 2;
-        for (int kg = 0; kg < kn / 4; ++kg) {
-            const float2 b = arow[kg * 4 * PA];
 #pragma unroll
-            for (int i = 0; i < NTW; ++i) {
-                const float2 a = *reinterpret_cast<const float2*>(wrow + kg * G::WGROUP + i * 64);
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[i], 0, 0, 0);
+        for (int i = 0; i < TPW; ++i) {
+            const int tile = tile0 + ((i + rot) & (TPW - 1));
+            const float* wrow = sW + kq * G::WROW + tile * 16 + col;
+#pragma unroll
+            for (int kg = 0; kg < KC / 4; ++kg) {
+                const float2 b = arow[kg * 4 * PA];
+                const float* w = wrow + kg * G::WGROUP;
+                p1[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0], b.x + b.y, p1[i], 0, 0, 0);
+                p2[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[G::WPLANE], b.x, p2[i], 0, 0, 0);
+                p3[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * G::WPLANE], b.y, p3[i], 0, 0, 0);
+            }
+            if (last) {
+                // D[row = 4 kq + v][col]: output channel n = 16 tile + 4 kq + v, mode 16 mt + col. NB is a multiple of
+                // 8, so the four channels of a lane have one owner.
+                const int n = 16 * tile + 4 * kq;
+                const bool own = n / NB == q;
+#pragma unroll
+                for (int vv = 0; vv < 4; ++vv) {
+                    const float2 c = make_float2(p1[i][vv] - p3[i][vv], p1[i][vv] + p2[i][vv]);
+                    if (own) sC[(n + vv - NB * q) * PC + mt * 16 + col] = c;
+                    else store_published(mine + (long)(n + vv) * 64, c);
+                }
             }
         }
-        __syncthreads();                                        // sA / sW are free again (next chunk, or sC below)
-    }
-
-    // D[row = 4 kq + v][col] of tile i: output channel n = 8 (nt0 + i) + 2 kq + (v >> 1), re | im = v & 1, mode 16 mt + col.
-    // NB is a multiple of 8, so the owner n / NB is the same for the whole tile.
-    {
-        float2* mine = part + ((long)(s * P + q) * N) * 64 + mt * 16 + col;
-#pragma unroll
-        for (int i = 0; i < NTW; ++i) {
-            const int n = 8 * (nt0 + i) + 2 * kq;
-            const float2 c0 = make_float2(acc[i][0], acc[i][1]), c1 = make_float2(acc[i][2], acc[i][3]);
-            if (n / NB == q) {
-                sC[(n - NB * q) * PC + mt * 16 + col] = c0;
-                sC[(n + 1 - NB * q) * PC + mt * 16 + col] = c1;
-            } else {
-                store_published(mine + (long)n * 64, c0);
-                store_published(mine + (long)(n + 1) * 64, c1);
-            }
-        }
+        if (!last) __syncthreads();                             // sA / sW are free again for the next chunk
     }
     stores_complete();
     __syncthreads();
     if (tid == 0) {
         unsigned* ctr = arrive + s * kArriveStride;
-        const unsigned old = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const unsigned target = (old / (unsigned)P + 1u) * (unsigned)P;     // P is a power of two: consistent under wrap-around
+        // every member adds 8 / P, every launch 8 whatever its cluster size: launches with different P may follow each
+        // other on a stream. 8 divides 2^32: consistent under wrap-around.
+        const unsigned old = __hip_atomic_fetch_add(ctr, 8u / (unsigned)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned target = (old / 8u + 1u) * 8u;
         if ((int)(counter_load(ctr) - target) < 0) {
             const unsigned long long t0 = wall_clock64();
             while ((int)(counter_load(ctr) - target) < 0) {
@@ -267,50 +279,55 @@ Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_clust
     return &e;
 }
 
-template <int NT>
+template <int NT, int KC>
 hipError_t launch_cluster_t(long S, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha, Exchange* e,
                             hipStream_t stream)
 {
-    using G = GeoCluster<NT>;
+    using G = GeoCluster<NT, KC>;
     static std::atomic<unsigned long long> served;
-    if (hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_cluster_kernel<NT>), G::LDS_BYTES, served);
+    if (hipError_t err = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_cluster_kernel<NT, KC>), G::LDS_BYTES, served);
         err != hipSuccess)
         return err;
     const long blocks = ((S + 7) / 8) * 8 * P;
-    hipLaunchKernelGGL(fused_fft_mfma_ifft_cluster_kernel<NT>, dim3((unsigned)blocks), dim3(512), G::LDS_BYTES, stream, (int)S, K, P,
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_cluster_kernel<NT, KC>), dim3((unsigned)blocks), dim3(512), G::LDS_BYTES, stream, (int)S, K, P,
                        x, W, y, alpha, e->part, e->arrive, e->gave_up, g_wait_ticks.load(std::memory_order_relaxed));
     return hipGetLastError();
 }
 
 }  // namespace
 
-// Cluster size for (S, N, K), or 0 when this kernel does not apply: N in {64, 128}, every member gets a multiple of four
+// Cluster size for (S, N, K), or 0 when this kernel does not apply: N in {64, 128}, every member gets a multiple of eight
 // input channels and 8 ... 32 output channels, and the whole grid is resident at once (one block per CU).
 int cluster_size_1d(int logDY, long S, int N, int K)
 {
     if (logDY != 8 || (N != 64 && N != 128) || S <= 0) return 0;
-    const long cus = cu_count();
-    int P = N / 32;
-    while (P < 8 && ((S + 7) / 8) * 8 * (2 * P) <= cus) P *= 2;
-    if (((S + 7) / 8) * 8 * P > cus) return 0;
-    if (K % (4 * P) != 0 || N / P < 8) return 0;
+    const long cus = cu_count(), groups = (S + 7) / 8 * 8;
+    int P = 0;
+    for (int c = N / 32; c <= 8; c *= 2)                        // the largest cluster that still gives every block a CU
+        if (groups * c <= cus && K % (8 * c) == 0 && N / c >= 8) P = c;
     return P;
 }
 
 // hipErrorNotReady: the exchange buffer could not be provided (the caller falls back on a kernel without one);
-// hipErrorLaunchFailure: an earlier launch on this stream gave up waiting for a cluster member.
+// hipErrorLaunchTimeOut: an earlier launch on this stream gave up waiting for a cluster member (reported once).
 hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
                                 hipStream_t stream)
 {
-    if (P < 2 || (P & (P - 1)) || K % (4 * P) || N % P || N / P > 32 || N / P < 8) return hipErrorInvalidValue;
+    if (P < 2 || P > 8 || (P & (P - 1)) || K % (8 * P) || N % P || N / P > 32 || N / P < 8) return hipErrorInvalidValue;
     Exchange* e = exchange_for(stream, S, sizeof(float2) * 64 * (size_t)N * P);
     if (!e) return hipErrorNotReady;
     if (*static_cast<volatile unsigned*>(e->gave_up)) {          // reported once; the arrival counters stay consistent
         *e->gave_up = 0;
-        return hipErrorLaunchFailure;
+        return hipErrorLaunchTimeOut;
     }
-    if (N == 128) return launch_cluster_t<128>(S, K, P, x, W, y, alpha, e, stream);
-    if (N == 64) return launch_cluster_t<64>(S, K, P, x, W, y, alpha, e, stream);
+    // chunk = the largest of 32 / 16 / 8 channels that divides a member's share
+    const int KB = K / P, KC = KB % 32 == 0 ? 32 : (KB % 16 == 0 ? 16 : 8);
+    if (N == 128 && KC == 32) return launch_cluster_t<128, 32>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 128 && KC == 16) return launch_cluster_t<128, 16>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 128) return launch_cluster_t<128, 8>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 64 && KC == 32) return launch_cluster_t<64, 32>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 64 && KC == 16) return launch_cluster_t<64, 16>(S, K, P, x, W, y, alpha, e, stream);
+    if (N == 64) return launch_cluster_t<64, 8>(S, K, P, x, W, y, alpha, e, stream);
     return hipErrorInvalidValue;
 }
 
