@@ -762,21 +762,22 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
     //    every K, even K = 8 where most of a chunk is padding;
     //  * grids of several items per SIMD: one wavefront per item (no barriers, nothing staged through LDS). At DY = 128
-    //    it is ahead for every K from about four items per CU; at DY = 256, where the block kernels are closer to
-    //    what the access pattern allows, from eight items per CU and not for 16 < K < 64;
-    //  * in between, K >= 32: matrix cores, 256-thread blocks, two or three per CU - the SIMT kernel is bound by
-    //    its vector instructions there, up to half of which are the contraction (lengths 512 / 1024: a tie within a
-    //    few percent for every K, the SIMT kernel stays; on small grids the 512-thread kernel is 30-40 % ahead there too);
-    //  * in between, K < 32: the SIMT kernel (three blocks per CU at DY = 256, two at DY = 128; no idle lanes in short
-    //    chunks; a tie at K = 16).
+    //    it is ahead from two (K <= 16), four (K < 128) or eight items per CU; at DY = 256, where the block kernels are
+    //    closer to what the access pattern allows, for K >= 128 (2-8 % from eight items per CU) and, K >= 24, on the
+    //    very largest grids (4-6 % from 128 items per CU); below that the 256-thread block kernel is level or up to
+    //    13 % ahead;
+    //  * otherwise: matrix cores, 256-thread blocks, two or three per CU, for every K - measured 5-27 % ahead of the
+    //    SIMT kernel on grids of 1 to 12 items per CU also for K < 32, where most of a chunk is padding (lengths
+    //    512 / 1024: a tie within a few percent for every K, the SIMT kernel stays; on small grids the 512-thread
+    //    kernel is 30-40 % ahead there too).
     const bool built = logDY >= 7 && logDY <= 10;
     const bool long_signal = logDY >= 9;            // 512 / 1024: on large grids the block kernels tie with the SIMT kernel
     const long items = S * (N / 64);
     if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
-    if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : 4) * (long)cu_count())
+    if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
         return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
-    if (algo == 0 && logDY == 8 && items >= 8L * cu_count() && (K <= 16 || K >= 64))
+    if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cu_count() : (K >= 24 && items >= 128L * cu_count())))
         return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     // small grids, 64 channels or more, N = 64 / 128: a cluster of blocks per signal set, no forward transform twice.
     // Without its exchange buffer (first use inside a stream capture, out of memory) the kernels below take over.
@@ -789,7 +790,7 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
     }
     int pick = algo == 4 ? 2 : algo;
-    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (K >= 32 && !long_signal ? 3 : 1);
+    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (!long_signal ? 3 : 1);
     // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
     // shares the spectra through LDS; level at K = 32)
     if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cu_count()))) {
