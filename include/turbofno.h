@@ -161,8 +161,7 @@ int turbofno_get_1d_algo(void);
  * Clustered launches (no counterpart in the reference). On small grids with K >= 64 (DY = 256, N = 64 or 128, every
  * block on a CU of its own) the fused 1D layer splits the K channels of a signal set over 2 - 8 blocks, which exchange
  * partial products through a device buffer that the library owns: one per (device, stream) that has used this path,
- * at most 512 N bytes per compute unit (16 MiB for N = 128 on 256 CUs), allocated on first use and kept until the
- * process ends. Consequences for callers:
+ * 64 KiB per compute unit (16 MiB on 256 CUs), allocated on first use, never moved, and kept until the process ends. Consequences for callers:
  *   - calls on one stream are ordered and share the buffer; calls on different streams use different buffers;
  *   - the first such call on a stream allocates (and synchronises the device once); inside a stream capture that is
  *     not possible, and a kernel without the exchange runs instead. A captured launch keeps using the buffer of the

@@ -222,8 +222,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// Exchange memory: one buffer per (device, stream) that has used this path, grown on demand and kept until the process
-// ends. Calls on one stream are ordered and may share it; calls on different streams get different buffers.
+// Exchange memory: one buffer per (device, stream) that has used this path, kept until the process ends. Calls on one stream are ordered and may share it; calls on different streams get different buffers.
 namespace {
 
 struct Exchange {
@@ -245,8 +244,10 @@ bool stream_is_capturing(hipStream_t stream)
     return st != hipStreamCaptureStatusNone;
 }
 
-// Returns the buffer of (current device, stream), sized for `clusters` signal sets of `bytes_per_cluster`; nullptr when
-// it cannot be provided (allocation failed, or it would have to be allocated while the stream is being captured).
+// Returns the buffer of (current device, stream); nullptr when it cannot be provided (allocation failed, or it would have
+// to be allocated while the stream is being captured). It is allocated once, at the largest size any launch can need
+// (a grid is at most one block per CU, N at most 128), and never freed or moved afterwards: a captured launch holds
+// its address.
 Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_cluster)
 {
     int dev = 0;
@@ -254,27 +255,33 @@ Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_clust
     std::lock_guard<std::mutex> lock(g_exchange_mutex);
     Exchange& e = g_exchange[{ dev, stream }];
     const size_t need = (size_t)clusters * bytes_per_cluster;
-    if (e.part_bytes >= need && e.clusters >= clusters && e.gave_up) return &e;
+    if (e.part && e.arrive && e.gave_up) return (e.part_bytes >= need && e.clusters >= clusters) ? &e : nullptr;
     if (stream_is_capturing(stream)) return nullptr;
+    const long cus = cu_count();
+    const size_t part_bytes = sizeof(float2) * 64 * 128 * (size_t)cus;          // part[S][P][N][64] with S P <= cus, N <= 128
+    const size_t arrive_bytes = sizeof(unsigned) * kArriveStride * (size_t)cus;
+    if (need > part_bytes || clusters > cus) return nullptr;
     if (!e.gave_up) {
-        if (hipHostMalloc(reinterpret_cast<void**>(&e.gave_up), 64, hipHostMallocDefault) != hipSuccess) { e.gave_up = nullptr; return nullptr; }
+        if (hipHostMalloc(reinterpret_cast<void**>(&e.gave_up), 64, hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            e.gave_up = nullptr;
+            return nullptr;
+        }
         *e.gave_up = 0;
     }
-    if (e.part_bytes < need) {
-        if (e.part) (void)hipFree(e.part);                      // hipFree waits for the work that may still use it
-        e.part = nullptr;
-        e.part_bytes = 0;
-        if (hipMalloc(reinterpret_cast<void**>(&e.part), need) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-        e.part_bytes = need;
+    if (!e.part) {
+        if (hipMalloc(reinterpret_cast<void**>(&e.part), part_bytes) != hipSuccess) { (void)hipGetLastError(); e.part = nullptr; return nullptr; }
+        e.part_bytes = part_bytes;
     }
-    if (e.clusters < clusters) {
-        if (e.arrive) (void)hipFree(e.arrive);
-        e.arrive = nullptr;
-        e.clusters = 0;
-        const size_t bytes = sizeof(unsigned) * kArriveStride * (size_t)clusters;
-        if (hipMalloc(reinterpret_cast<void**>(&e.arrive), bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-        if (hipMemset(e.arrive, 0, bytes) != hipSuccess) return nullptr;      // synchronous, once per growth
-        e.clusters = clusters;
+    if (!e.arrive) {
+        if (hipMalloc(reinterpret_cast<void**>(&e.arrive), arrive_bytes) != hipSuccess) { (void)hipGetLastError(); e.arrive = nullptr; return nullptr; }
+        if (hipMemset(e.arrive, 0, arrive_bytes) != hipSuccess) {                // synchronous, once
+            (void)hipGetLastError();
+            (void)hipFree(e.arrive);
+            e.arrive = nullptr;
+            return nullptr;
+        }
+        e.clusters = cus;
     }
     return &e;
 }
