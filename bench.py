@@ -37,6 +37,10 @@ def main():
               "multi-GPU runs are not part of it). Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
+    # ROCm runtime knob, read when HIP initialises: kernel arguments are placed in device memory instead of host memory,
+    # which takes about a microsecond off the start of every kernel (measured on the layer: 226.0 -> 223.6 us). A setting
+    # already present in the environment wins; the value in force is reported in the JSON line.
+    os.environ.setdefault("HIP_FORCE_DEV_KERNARG", "1")
     import torch
     import turbofno_amd as tf
     from turbofno_amd import workloads
@@ -212,6 +216,7 @@ def main():
         "config": {"workload": "2D layer bs=%d 256x256 K=64 N=64, 64x64 modes, Gaussian random field input" % bs,
                    "algo": ("auto -> " if args.algo == 0 else "") + {1: "three-kernel", 2: "whole-image"}[algo]},
         "settle": {"ms": args.settle_ms, "steps": settle_steps},
+        "env": {"HIP_FORCE_DEV_KERNARG": os.environ.get("HIP_FORCE_DEV_KERNARG")},
         "layer_algorithmic_bytes": layer_bytes, "layer_GBps": round(layer_gbs, 1),
         "layer_hbm_frac": round(layer_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall_ms, 4),
         "stage_ms": {k: round(v, 4) for k, v in stages.items()},

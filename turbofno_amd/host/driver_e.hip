@@ -57,6 +57,9 @@ struct Problem { int bs, dx, dy, n, k; };
 
 int main(int argc, char** argv)
 {
+    // kernel arguments in device memory (ROCm runtime knob, read when HIP initialises; an existing setting wins):
+    // about a microsecond less at the start of every kernel
+    setenv("HIP_FORCE_DEV_KERNARG", "1", 0);
     std::vector<Problem> problems;
     if (argc == 6) problems.push_back({ atoi(argv[1]), atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]) });
     else {
