@@ -25,8 +25,11 @@
 #include "group_fft.h"
 #include "kernels.h"
 
+#include <functional>
 #include <map>
 #include <mutex>
+#include <thread>
+#include <tuple>
 
 namespace tfno {
 
@@ -234,7 +237,9 @@ struct Exchange {
 };
 
 std::mutex g_exchange_mutex;
-std::map<std::pair<int, hipStream_t>, Exchange> g_exchange;
+// key: device, stream handle, and - for hipStreamPerThread, one handle that names a different stream in every host
+// thread - a hash of the calling thread
+std::map<std::tuple<int, hipStream_t, size_t>, Exchange> g_exchange;
 std::atomic<unsigned long long> g_wait_ticks{ 200000000ull };    // 2 s of the 100 MHz wall clock
 
 bool stream_is_capturing(hipStream_t stream)
@@ -253,7 +258,8 @@ Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_clust
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lock(g_exchange_mutex);
-    Exchange& e = g_exchange[{ dev, stream }];
+    const size_t thread_key = stream == hipStreamPerThread ? std::hash<std::thread::id>()(std::this_thread::get_id()) : 0;
+    Exchange& e = g_exchange[std::make_tuple(dev, stream, thread_key)];
     const size_t need = (size_t)clusters * bytes_per_cluster;
     if (e.part && e.arrive && e.gave_up) return (e.part_bytes >= need && e.clusters >= clusters) ? &e : nullptr;
     if (stream_is_capturing(stream)) return nullptr;
