@@ -50,6 +50,8 @@ extern "C" {
  * M = 64 * S where S = bs*dimX signals per channel. `C` is unused by the reference kernel (its beta*C
  * term is commented out, fused_fft_cgemm_ifft_7.cuh:186-187) and may be NULL; beta is ignored.
  * Requires logDY in {7, 8, 9, 10}, M % 64 == 0, N % 64 == 0, K % 8 == 0 (utils/TurboFNO.h:2-4).
+ * On small grids with K >= 64 this entry point and turbofno_layer_1d may use a library-owned exchange buffer and
+ * return TURBOFNO_ERR_EXCHANGE: see "Clustered launches" below.
  */
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
