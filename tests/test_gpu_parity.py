@@ -257,3 +257,34 @@ def test_image_stage_entry_points(DX, DY, tol):
     padded = np.zeros((nimg, DX, DY), dtype=np.complex128)
     padded[:, :64, :64] = modes
     check(y, np.fft.ifft2(padded, axes=(1, 2)) * (DX * DY), tol, "ifft2d_pad")
+
+
+def test_layer_1d_across_the_size_rule():
+    """60 seeded shapes from one signal set to a few items per CU (S up to 700, all four lengths, K up to 136, N up to
+    256), kernel chosen by size: crosses every branch of the choice (clustered, 512- and 256-thread blocks, one
+    wavefront per item, SIMT for the long lengths). The oracle takes minutes at these sizes, so the comparison is with
+    an fp64 evaluation of the same definition by torch.fft / einsum on the GPU (the oracle itself is pinned to
+    numpy.fft and covers the small shapes above)."""
+    rng = np.random.default_rng(20251)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    for it in range(60):
+        DY = int(rng.choice([128, 256, 256, 256, 512, 1024]))
+        K = 8 * int(rng.integers(1, 18))
+        N = 64 * int(rng.integers(1, 5)) if rng.random() < 0.3 else int(rng.choice([64, 128]))
+        S = int(rng.integers(1, 700)) if rng.random() < 0.5 else int(rng.integers(1, 70))
+        if DY >= 512:
+            S = min(S, 200)
+        alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
+        print("case size rule", it, "S", S, "DY", DY, "K", K, "N", N, flush=True)
+        x = torch.complex(torch.rand((K, S, DY), generator=gen, device="cuda") - 0.5,
+                          torch.rand((K, S, DY), generator=gen, device="cuda") - 0.5)
+        W = torch.complex(torch.rand((N, K), generator=gen, device="cuda") - 0.5,
+                          torch.rand((N, K), generator=gen, device="cuda") - 0.5)
+        y = tf.layer_1d(x, W, alpha=alpha).to(torch.complex128)
+        spec = torch.fft.fft(x.to(torch.complex128), dim=-1)[..., :64]
+        padded = torch.zeros((N, S, DY), dtype=torch.complex128, device="cuda")
+        padded[..., :64] = alpha * torch.einsum("ksm,nk->nsm", spec, W.to(torch.complex128))
+        ref = torch.fft.ifft(padded, dim=-1) * DY                    # unnormalised backward transform
+        err = float(torch.linalg.vector_norm(y - ref) / torch.linalg.vector_norm(ref))
+        worst = float((y - ref).abs().max() / ref.abs().max())
+        assert err <= 1e-5 and worst <= 1e-4, (it, S, DY, K, N, err, worst)
