@@ -84,7 +84,7 @@ def test_1d_kernel_selector_round_trip():
     prev = tf.set_1d_algo(5)
     assert tf.lib().turbofno_get_1d_algo() == 5
     with pytest.raises(tf.TurboFNOError):
-        tf.set_1d_algo(8)
+        tf.set_1d_algo(9)
     assert tf.lib().turbofno_get_1d_algo() == 5           # a refused value changes nothing
     tf.set_1d_algo(prev)
 

@@ -51,7 +51,7 @@ def test_config2_sweep_against_oracle(tol):
 
 
 @pytest.mark.parametrize("K", [64, 128])
-@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 def test_config3_large_hidden_against_oracle(K, algo, tol, algo_1d):
     """1D bs=64, DY=256, N=128, K in {64, 128}, smooth input: size-chosen kernel, SIMT kernel, the three matrix-core variants"""
     print("config3", K, algo, flush=True)

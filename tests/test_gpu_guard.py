@@ -24,7 +24,7 @@ def intact(buf, what):
     assert bool((lo == CANARY).all()) and bool((hi == CANARY).all()), what + ": guard band overwritten"
 
 
-@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("bs,DY,K,N", [(3, 256, 72, 128), (5, 128, 40, 64), (1, 256, 8, 64), (7, 128, 136, 128),
                                        (5, 256, 64, 128), (13, 256, 192, 64)])
 def test_layer_1d_stays_in_bounds(bs, DY, K, N, algo, algo_1d):

@@ -47,7 +47,7 @@ def test_layer_1d(bs, DY, K, N, alpha, tol):
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d")
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("bs,DY,K,N,alpha", [
     (2, 256, 32, 64, 1.0),           # exactly one chunk of the matrix-core kernel
     (3, 256, 72, 128, 1 - 1j),       # chunks 32 + 32 + 8, two N tiles
@@ -66,7 +66,7 @@ def test_layer_1d_both_contractions(bs, DY, K, N, alpha, algo, tol, algo_1d):
     check(y, oracle.layer_1d(x, W, alpha), tol, "layer_1d algo %d" % algo)
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(36))
 def test_layer_1d_random_shapes(seed, tol, algo_1d):
     """seeded random shapes (odd S, three N tiles, K up to 136, complex alpha) through every 1D kernel choice"""
     rng = np.random.default_rng(1000 + seed)
@@ -74,7 +74,7 @@ def test_layer_1d_random_shapes(seed, tol, algo_1d):
     K = 8 * int(rng.integers(1, 18))
     N = 64 * int(rng.integers(1, 4))
     S = int(rng.integers(1, 41))
-    algo = seed % 8
+    algo = seed % 9
     alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
     print("case layer_1d random", seed, "S", S, "DY", DY, "K", K, "N", N, "algo", algo, flush=True)
     algo_1d(algo)

@@ -75,7 +75,8 @@ const char* turbofno_last_error_string(void) { return g_err; }
 // the process-wide selector set by turbofno_set_1d_algo (0 by size, 1 SIMT contraction, 2 / 3 matrix cores with
 // 512- / 256-thread blocks, 4 matrix cores with 512 threads and 32-channel output tiles, 5 matrix cores with one
 // wavefront per signal set and output tile, 6 matrix cores with the K channels of an item split over the waves of a
-// block, 7 matrix cores with the K channels of a signal set split over a cluster of blocks) overrides the choice by size.
+// block, 7 matrix cores with the K channels of a signal set split over a cluster of blocks, 8 matrix cores with tiles of
+// 128 output channels) overrides the choice by size.
 static std::atomic<int> g_algo_1d{ 0 };
 static int algo_1d() { return g_algo_1d.load(std::memory_order_relaxed); }
 

@@ -14,6 +14,27 @@ namespace tfno {
 constexpr int kWHalf = 516;
 constexpr int kWGroup = 1032;
 
+#ifdef __HIPCC__
+// Block -> (signal set s, output tile) for the fused 1D kernels. Consecutive workgroups go to different XCDs (eight L2s),
+// and every output tile of a signal set re-reads the same K input rows: the tiles of one s are therefore given block
+// ids eight apart, which lands them on the same XCD at about the same time, so only the first of them reads x from
+// HBM. Groups of eight signal sets are laid out as [tile][s % 8]; a tail of fewer than eight sets is laid out plainly.
+__device__ __forceinline__ void decode_block_1d(long S, int ntiles, long& s, int& tile)
+{
+    const long id = blockIdx.x, full = (S / 8) * 8;
+    if (id < full * ntiles) {
+        const long grp = id / (8 * ntiles);
+        const int rem = (int)(id % (8 * ntiles));
+        tile = rem / 8;
+        s = grp * 8 + rem % 8;
+    } else {
+        const long rem = id - full * ntiles;
+        s = full + rem / ntiles;
+        tile = (int)(rem % ntiles);
+    }
+}
+#endif
+
 // compute units of the current device (cached per device)
 int cu_count();
 
@@ -44,6 +65,10 @@ int cluster_size_1d(int logDY, long S, int N, int K);
 hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
                                 hipStream_t stream);
 void set_cluster_wait_ticks(unsigned long long ticks);
+
+// Large grids, DY = 256 (layer1d_wide.hip): one block per (signal set, 128 or 64 output channels), three-real-product
+// contraction.
+hipError_t launch_fused_wide(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha, hipStream_t stream);
 
 // Halves of the fused kernel (variants B and C) and the stand-alone contiguous transforms (variant A).
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

@@ -16,25 +16,6 @@
 
 namespace tfno {
 
-// Block -> (signal set s, output tile) for the fused 1D kernels. Consecutive workgroups go to different XCDs (eight L2s),
-// and every output tile of a signal set re-reads the same K input rows: the tiles of one s are therefore given block
-// ids eight apart, which lands them on the same XCD at about the same time, so only the first of them reads x from
-// HBM. Groups of eight signal sets are laid out as [tile][s % 8]; a tail of fewer than eight sets is laid out plainly.
-__device__ __forceinline__ void decode_block_1d(long S, int ntiles, long& s, int& tile)
-{
-    const long id = blockIdx.x, full = (S / 8) * 8;
-    if (id < full * ntiles) {
-        const long grp = id / (8 * ntiles);
-        const int rem = (int)(id % (8 * ntiles));
-        tile = rem / 8;
-        s = grp * 8 + rem % 8;
-    } else {
-        const long rem = id - full * ntiles;
-        s = full + rem / ntiles;
-        tile = (int)(rem % ntiles);
-    }
-}
-
 // FUSE_FWD: the A operand is produced by forward transforms of x (variants B and D); otherwise it is read from
 //           the column-major matrix A[m + k*M] (variant C).
 // FUSE_INV: the product goes straight into zero-padded backward transforms (variants C and D); otherwise it is
@@ -754,7 +735,8 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
 // algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
 // 4 = as 2 with 32-channel output tiles, 5 = matrix cores, one wavefront per (signal set, output tile),
 // 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256),
-// 7 = matrix cores, a cluster of blocks splits the K channels of one signal set (DY = 256, N = 64 / 128, small grids)
+// 7 = matrix cores, a cluster of blocks splits the K channels of one signal set (DY = 256, N = 64 / 128, small grids),
+// 8 = matrix cores, 256-thread blocks with tiles of 128 output channels, three real products per complex one (DY = 256)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream)
 {
@@ -775,6 +757,14 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     const long items = S * (N / 64);
     if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
     if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
+    // N a multiple of 128, DY = 256, K >= 16: blocks with tiles of 128 output channels (every input channel transformed
+    // once per signal set, three real products per complex one): 5-20 % ahead of the kernels below on every grid that
+    // fills its two slots per CU reasonably evenly (measured from 400 blocks up; with a last round under three quarters
+    // full the 64-channel kernels, with their finer blocks, are ahead)
+    if (algo == 0 && logDY == 8 && N % 128 == 0 && K >= 16) {
+        const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
+        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(S, N, K, x, W, y, alpha, stream);
+    }
     if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
         return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
     if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cu_count() : (K >= 24 && items >= 128L * cu_count())))
@@ -789,6 +779,8 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         }
         if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
     }
+    if (algo == 8 && logDY == 8) return launch_fused_wide(S, N, K, x, W, y, alpha, stream);
+    if (algo == 8) algo = 0;
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (!long_signal ? 3 : 1);
     // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
