@@ -154,7 +154,7 @@ int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* 
  * 32-channel output tiles, 5 = matrix cores, one wavefront per signal set and output tile, 6 = matrix cores, the K
  * channels of an item split over the waves of a block, 7 = matrix cores, the K channels of a signal set split over a
  * cluster of blocks (see below), 8 = matrix cores, 256-thread blocks with tiles of 128 output channels and three real
- * products per complex one (DY = 256). A value a kernel is not built for falls back to the choice by size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
+ * products per complex one (DY = 128 / 256). A value a kernel is not built for falls back to the choice by size. Meant for tests and measurements; set returns TURBOFNO_ERR_INVALID_ARG outside 0..TURBOFNO_1D_ALGO_MAX.
  */
 #define TURBOFNO_1D_ALGO_MAX 8
 int turbofno_set_1d_algo(int algo);

@@ -66,9 +66,10 @@ hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, co
                                 hipStream_t stream);
 void set_cluster_wait_ticks(unsigned long long ticks);
 
-// Large grids, DY = 256 (layer1d_wide.hip): one block per (signal set, 128 or 64 output channels), three-real-product
+// Large grids, DY = 128 / 256 (layer1d_wide.hip): one block per (signal set, 128 or 64 output channels), three-real-product
 // contraction.
-hipError_t launch_fused_wide(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha, hipStream_t stream);
+hipError_t launch_fused_wide(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                             hipStream_t stream);
 
 // Halves of the fused kernel (variants B and C) and the stand-alone contiguous transforms (variant A).
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

@@ -763,7 +763,14 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     // full the 64-channel kernels, with their finer blocks, are ahead)
     if (algo == 0 && logDY == 8 && N % 128 == 0 && K >= 16) {
         const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
-        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(S, N, K, x, W, y, alpha, stream);
+        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream);
+    }
+    // the same at DY = 128 for K >= 64 (3-21 % ahead up to 64 blocks per CU; with fewer channels, or on the very largest
+    // grids, the one-wavefront kernel below is level or ahead)
+    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 64) {
+        const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
+        if (blocks > cu_count() && blocks <= 64L * cu_count() && 4 * blocks >= 3 * rounds * slots)
+            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream);
     }
     if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
         return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
@@ -779,7 +786,7 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         }
         if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
     }
-    if (algo == 8 && logDY == 8) return launch_fused_wide(S, N, K, x, W, y, alpha, stream);
+    if (algo == 8 && (logDY == 7 || logDY == 8)) return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream);
     if (algo == 8) algo = 0;
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (!long_signal ? 3 : 1);

@@ -1,4 +1,4 @@
-// Fused 1D spectral layer for LARGE grids with many channels (DY = 256): one 256-thread block per (signal set, NT output
+// Fused 1D spectral layer for LARGE grids with many channels (DY = 256, and DY = 128 further down): one 256-thread block per (signal set, NT output
 // channels) with NT = 128 or 64, so that with N = 128 every input channel of a signal set is transformed once, not once
 // per 64 output channels, and the contraction takes three real matrix instructions per complex product instead of four.
 //
@@ -147,22 +147,163 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide_kernel(int S,
     }
 }
 
+// The same for DY = 128, where a 16-lane group transforms two channels at a time (pair128_forward / _backward), so that a
+// round of the block covers 32 channels: the spectra tile holds 32 channels, the W'' tile 16 - it is built and multiplied
+// twice per round, and the rows of W for the second half are fetched while the first half is being multiplied. The
+// product goes to LDS 32 channels at a time.
 template <int NT>
-static hipError_t launch_wide_t(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha, hipStream_t stream)
+__global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide128_kernel(int S, int N, int K, const float2* __restrict__ x,
+                                                                            const float2* __restrict__ W, float2* __restrict__ y,
+                                                                            float2 alpha)
+{
+    using G = GeoWide<NT>;
+    constexpr int DY = 128, PA = G::PA, PC = G::PC, TILES = G::TILES, KR = 32;    // KR = channels per round
+    static_assert(KR * PA <= G::REGION0 && KR * PC <= G::REGION1, "32-channel tiles must fit the regions");
+    extern __shared__ float2 lds[];
+    float2* sA = lds;
+    float* sW = reinterpret_cast<float*>(lds + G::REGION0);
+    float2* sC = lds + G::REGION0;
+
+    const int tid = threadIdx.x;
+    const int grp = tid >> 4, t16 = tid & 15;                   // transform role: 16-lane group, two channels each
+    const int g8 = tid >> 3, r8 = tid & 7;                      // after the exchange: lane r8 of channel g8 of the round
+    const int mt = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;     // matrix role: m tile = wave
+    long s;
+    int ntile;
+    decode_block_1d(S, N / NT, s, ntile);
+    const int n0 = ntile * NT;
+    float2* exch = lds + grp * G::EXCH;
+
+    cpx tw[16];
+    load_lane_twiddles<7>(t16, tw);
+    floatx4_w p1[TILES], p2[TILES], p3[TILES];
+#pragma unroll
+    for (int i = 0; i < TILES; ++i) p1[i] = p2[i] = p3[i] = floatx4_w{ 0.f, 0.f, 0.f, 0.f };
+
+    const float2* src = x + ((long)(2 * grp) * S + s) * DY + t16;
+    auto issue = [&](cpx (&dst)[16], int kc) {
+        const float2* p = src + (long)kc * S * DY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { dst[i] = p[16 * i]; dst[8 + i] = p[(long)S * DY + 16 * i]; }
+    };
+    cpx v[16];
+    if (2 * grp < K) issue(v, 0);
+
+    constexpr int WPT = 16 * NT / 256;
+    auto load_w = [&](float2 (&wv)[WPT], int k0, int kn) {      // rows k0 ... k0 + 15 of W, zeros from row kn of the round on
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * 256;
+            const int k = idx % 16, r = idx / 16, n = (r & ~15) | ((r & 3) << 2) | ((r >> 2) & 3);
+            wv[u] = (k0 % KR + k < kn) ? W[(k0 + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        }
+    };
+    auto build_w = [&](const float2 (&wv)[WPT]) {
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * 256;
+            const int k = idx % 16, r = idx / 16, n = (r & ~15) | ((r & 3) << 2) | ((r >> 2) & 3);
+            const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+            float* dstw = &sW[(k >> 2) * G::WGROUP + (k & 3) * G::WROW + n];
+            dstw[0] = c;
+            dstw[G::WPLANE] = d - c;
+            dstw[2 * G::WPLANE] = c + d;
+        }
+    };
+    auto multiply = [&](int half) {                             // channels 16 half ... 16 half + 15 of the round
+        const float2* arow = sA + (16 * half + kq) * PA + mt * 16 + col;
+        float2 b[4];
+#pragma unroll
+        for (int kg = 0; kg < 4; ++kg) b[kg] = arow[kg * 4 * PA];
+#pragma unroll
+        for (int i = 0; i < TILES; ++i) {
+            const float* wrow = sW + kq * G::WROW + i * 16 + col;
+#pragma unroll
+            for (int kg = 0; kg < 4; ++kg) {
+                const float* w = wrow + kg * G::WGROUP;
+                p1[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0], b[kg].x + b[kg].y, p1[i], 0, 0, 0);
+                p2[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[G::WPLANE], b[kg].x, p2[i], 0, 0, 0);
+                p3[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * G::WPLANE], b[kg].y, p3[i], 0, 0, 0);
+            }
+        }
+    };
+
+    for (int kc = 0; kc < K; kc += KR) {
+        const int kn = (K - kc) < KR ? (K - kc) : KR;           // 8, 16, 24 or 32 (K is a multiple of 8)
+        float2 wv[WPT];
+        load_w(wv, kc, kn);
+        cpx out[8];
+        if (2 * grp < kn) {
+            cpx w[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) w[i] = v[i];
+            if (kc + KR + 2 * grp < K) issue(v, kc + KR);
+            pair128_forward(w, tw, exch, t16, out);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) out[c] = make_float2(0.f, 0.f);
+        }
+        build_w(wv);
+        if (kn > 16) load_w(wv, kc + 16, kn);                   // second half of the rows: arrives under the first multiply
+        __syncthreads();                                        // all exchanges done: sA may overwrite them
+#pragma unroll
+        for (int c = 0; c < 8; ++c) sA[g8 * PA + r8 + 8 * c] = out[c];     // zeros beyond a short last round
+        __syncthreads();
+        multiply(0);
+        if (kn > 16) {                                          // uniform
+            __syncthreads();                                    // the first half of the W'' tile is consumed
+            build_w(wv);
+            __syncthreads();
+            multiply(1);
+        }
+        __syncthreads();                                        // sA / sW are free again (next round, or the product below)
+    }
+
+    // product -> LDS 32 channels (two tiles) at a time; lane (g8, r8) takes modes r8 + 8 k of channel 32 step + g8
+#pragma unroll
+    for (int step = 0; step < TILES / 2; ++step) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int vv = 0; vv < 4; ++vv) {
+                const int i = 2 * step + j;
+                sC[(16 * j + 4 * kq + vv) * PC + mt * 16 + col] = make_float2(p1[i][vv] - p3[i][vv], p1[i][vv] + p2[i][vv]);
+            }
+        __syncthreads();
+        cpx c[8], yv[16];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) c[k] = sC[g8 * PC + r8 + 8 * k];
+        __syncthreads();                                        // the buffer is consumed: the next step may overwrite it
+        pair128_backward(c, tw, exch, t16, yv);
+        float2* dst = y + ((long)(n0 + 32 * step + 2 * grp) * S + s) * DY + t16;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
+    }
+}
+
+template <int NT>
+static hipError_t launch_wide_t(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                hipStream_t stream)
 {
     using G = GeoWide<NT>;
     if (S * (N / NT) > 0x7fffffffL) return hipErrorInvalidValue;
     static_assert(G::LDS_BYTES <= 64 * 1024, "no attribute call needed below 64 KiB of dynamic LDS");
-    hipLaunchKernelGGL(fused_fft_mfma_ifft_wide_kernel<NT>, dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream, (int)S, N,
-                       K, x, W, y, alpha);
+    if (logDY == 7)
+        hipLaunchKernelGGL(fused_fft_mfma_ifft_wide128_kernel<NT>, dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream,
+                           (int)S, N, K, x, W, y, alpha);
+    else
+        hipLaunchKernelGGL(fused_fft_mfma_ifft_wide_kernel<NT>, dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream, (int)S,
+                           N, K, x, W, y, alpha);
     return hipGetLastError();
 }
 
-// DY = 256 only. Tiles of 128 output channels when N allows, else of 64.
-hipError_t launch_fused_wide(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha, hipStream_t stream)
+// DY = 128 or 256. Tiles of 128 output channels when N allows, else of 64.
+hipError_t launch_fused_wide(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                             hipStream_t stream)
 {
-    if (N % 128 == 0) return launch_wide_t<128>(S, N, K, x, W, y, alpha, stream);
-    return launch_wide_t<64>(S, N, K, x, W, y, alpha, stream);
+    if (logDY != 7 && logDY != 8) return hipErrorInvalidValue;
+    if (N % 128 == 0) return launch_wide_t<128>(logDY, S, N, K, x, W, y, alpha, stream);
+    return launch_wide_t<64>(logDY, S, N, K, x, W, y, alpha, stream);
 }
 
 }  // namespace tfno
