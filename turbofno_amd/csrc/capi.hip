@@ -53,14 +53,17 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // AUTO: the whole-image path runs one persistent block per image, so it needs enough input images (K*bs) to occupy
 // the CUs; below that the three-kernel path spreads an image over many blocks and is faster although it moves 1.5x
 // the bytes. Measured crossover on MI355X (256 CUs): one input image per CU, and for images smaller than 256 x 256
-// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner).
-int pick_algo(int bs, int DX, int DY, int K, int algo)
+// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner). Half an input image per
+// CU is enough when the output side is large (two output images per CU): the backward kernel, which writes most of the
+// bytes, then runs on a full grid (bs = 8, K = 16: 91 vs 100 us at N = 64, 140 vs 175 us at N = 128, 256 x 256).
+int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (algo != TURBOFNO_2D_AUTO) return algo;
     if (DX > 256 || DY > 256) return TURBOFNO_2D_THREE_KERNEL;      // an image no longer fits one block's LDS
-    const long images = (long)K * bs;
+    const long in_images = (long)K * bs, out_images = (long)N * bs;
     const bool big = DX == 256 && DY == 256;
-    return (images >= 256 && (big || bs >= 8)) ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
+    const bool enough = in_images >= 256 || (in_images >= 128 && out_images >= 512);
+    return (enough && (big || bs >= 8)) ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
 }
 
 }  // namespace
@@ -222,7 +225,7 @@ int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, co
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
-    if (pick_algo(bs, DX, DY, K, algo) == TURBOFNO_2D_WHOLE_IMAGE)
+    if (pick_algo(bs, DX, DY, K, N, algo) == TURBOFNO_2D_WHOLE_IMAGE)
         return align256((size_t)K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
     return align256((size_t)K * bs * 64 * DY * sizeof(float2)) + align256((size_t)N * bs * 64 * DY * sizeof(float2));
 }
@@ -246,7 +249,7 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
         return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
     if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the whole-image path is built for lengths in {128, 256}", DX, DY);
-    const int a = pick_algo(bs, DX, DY, K, algo);
+    const int a = pick_algo(bs, DX, DY, K, N, algo);
     const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
     if (!workspace || workspace_bytes < need)
         return fail(TURBOFNO_ERR_WORKSPACE, "%s of %zu bytes required, %zu available", what, need, workspace ? workspace_bytes : (size_t)0);
