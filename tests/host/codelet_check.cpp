@@ -153,9 +153,16 @@ template <int LOGD> static double check_wide(bool backward)
     } else {
         for (int m = 0; m < 64; ++m) exch[m] = make_float2((float)frand(), (float)frand());
         std::vector<cpx> y(D);
+        // first pass inputs as the kernels produce them: every lane's partial products, the second exchange, one row each
+        std::vector<cpx> modes(exch.begin(), exch.begin() + 64), rows(L * 17);
+        for (int l = 0; l < L; ++l) {
+            cpx part[16];
+            wide_backward_partial<L>(modes.data(), 1, l, part);
+            for (int k = 0; k < 16; ++k) rows[wide_back_index<L>(l, k)] = part[k];
+        }
         for (int t = 0; t < L; ++t) {
             cpx e[16], tw[16], out[16];
-            wide_backward_inputs<L>(exch.data(), t, e);
+            for (int r = 0; r < 16; ++r) e[r] = rows[t * 17 + r];
             load_lane_twiddles<LOGD>(t, tw);
             inv_pass2(e, tw, out);
             for (int i = 0; i < 16; ++i) y[t + L * i] = out[i];

@@ -347,14 +347,35 @@ template <int L> TFNO_DEV void wide_forward_outer(const cpx* swap, int es, int l
         out[j] = acc;
     }
 }
-// Backward: first-pass input r of lane t:  e[r] = sum_{c<4} C[r + 16 c] * conj(w_L^(t c)), C = exch[0..63].
-template <int L> TFNO_DEV void wide_backward_inputs(const cpx* exch, int t, cpx (&e)[16])
+// Backward: first-pass input r of lane t is  e[r] = sum_{c<4} C[r + 16 c] * conj(w_L^(t c)),  C = the 64 retained modes.
+// With t = t1 + (L/4) t2 the factor splits into conj(w_L^(t1 c)) * i^(t2 c): lane l = (t1 = l % (L/4), rq = l / (L/4))
+// twiddles the four modes C[r + 16 c] of r = rq + 4 ri, ri < 4, once (3 complex multiplications per r) and a 4-point
+// transform without multiplications gives the inputs of the four lanes t2 < 4 at once. part[4 ri + t2] then belongs to
+// lane t1 + (L/4) t2, slot r: the caller parks it at wide_back_index<L>(l, 4 ri + t2) of a pitch-17 array [L][17] (after
+// every lane has read C, which may live in the same array) and each lane reads its e[r] back from row t. 16 + 16 + 16
+// exchange accesses and ~110 flops per lane instead of 64 reads and ~290 flops for the direct sums.
+template <int L> TFNO_DEV void wide_backward_partial(const cpx* c64, int es, int l, cpx (&part)[16])
 {
-    const cpx w1 = kTwiddle1024[(t * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t * (1024 / L)) & 1023],
-              w3 = kTwiddle1024[(3 * t * (1024 / L)) & 1023];
+    constexpr int Q = L / 4;
+    const int t1 = l % Q, rq = l / Q;
+    const cpx w1 = kTwiddle1024[(t1 * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t1 * (1024 / L)) & 1023],
+              w3 = kTwiddle1024[(3 * t1 * (1024 / L)) & 1023];
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-        e[r] = cadd(cadd(exch[r], cmulc(exch[r + 16], w1)), cadd(cmulc(exch[r + 32], w2), cmulc(exch[r + 48], w3)));
+    for (int ri = 0; ri < 4; ++ri) {
+        const int r = rq + 4 * ri;
+        const cpx d0 = c64[r * es], d1 = cmulc(c64[(r + 16) * es], w1), d2 = cmulc(c64[(r + 32) * es], w2),
+                  d3 = cmulc(c64[(r + 48) * es], w3);
+        const cpx s02 = cadd(d0, d2), m02 = csub(d0, d2), s13 = cadd(d1, d3), m13 = csub(d1, d3);
+        const cpx im13 = make_float2(-m13.y, m13.x);            // i * (d1 - d3)
+        part[4 * ri + 0] = cadd(s02, s13);
+        part[4 * ri + 1] = cadd(m02, im13);
+        part[4 * ri + 2] = csub(s02, s13);
+        part[4 * ri + 3] = csub(m02, im13);
+    }
+}
+template <int L> TFNO_DEV constexpr int wide_back_index(int l, int k)
+{
+    return ((l % (L / 4)) + (L / 4) * (k & 3)) * 17 + (l / (L / 4)) + 4 * (k >> 2);
 }
 
 // Orders LDS traffic of one wavefront: everything the wave wrote before is visible to its own

@@ -100,7 +100,14 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
     wave_lds_fence();
     cpx e[16];
     if constexpr (L >= 32) {
-        wide_backward_inputs<L>(exch, t, e);
+        cpx part[16];
+        wide_backward_partial<L>(exch, 1, t, part);
+        wave_lds_fence();                               // every lane of the group has read the 64 modes
+#pragma unroll
+        for (int k = 0; k < 16; ++k) exch[wide_back_index<L>(t, k)] = part[k];
+        wave_lds_fence();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
     } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];

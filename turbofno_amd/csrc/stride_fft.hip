@@ -123,13 +123,16 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
     __syncthreads();
     cpx e[16], yv[16];
     if constexpr (L >= 32) {
-        // first-pass input r of row group t from the 64 retained rows (wide_backward_inputs on this layout)
-        const cpx w1 = kTwiddle1024[(t * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t * (1024 / L)) & 1023],
-                  w3 = kTwiddle1024[(3 * t * (1024 / L)) & 1023];
+        // first-pass inputs from the 64 retained rows: twiddle once per four row groups, 4-point transform, second small
+        // exchange (wide_backward_partial / wide_back_index on this kernel's [.][yl] layout)
+        cpx part[16];
+        wide_backward_partial<L>(lds + yl, COLS, t, part);
+        __syncthreads();                                 // every thread has read the 64 rows
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-            e[r] = cadd(cadd(lds[r * COLS + yl], cmulc(lds[(r + 16) * COLS + yl], w1)),
-                        cadd(cmulc(lds[(r + 32) * COLS + yl], w2), cmulc(lds[(r + 48) * COLS + yl], w3)));
+        for (int k = 0; k < 16; ++k) lds[wide_back_index<L>(t, k) * COLS + yl] = part[k];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * COLS + yl];
     } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * COLS + yl];
