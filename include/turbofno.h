@@ -83,8 +83,7 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:133-172). The reference keeps its
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
- * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE once the K*bs input images (or, from half of that, the N*bs output images)
- * fill the CUs, THREE_KERNEL below; the workspace query
+ * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE once K*bs images fill the CUs, THREE_KERNEL below; the workspace query
  * with the same arguments makes the same choice.
  */
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo);

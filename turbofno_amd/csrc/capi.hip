@@ -53,16 +53,17 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // AUTO: the whole-image path runs one persistent block per image, so it needs enough input images (K*bs) to occupy
 // the CUs; below that the three-kernel path spreads an image over many blocks and is faster although it moves 1.5x
 // the bytes. Measured crossover on MI355X (256 CUs): one input image per CU, and for images smaller than 256 x 256
-// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner). Half an input image per
-// CU is enough when the output side is large (two output images per CU): the backward kernel, which writes most of the
-// bytes, then runs on a full grid (bs = 8, K = 16: 91 vs 100 us at N = 64, 140 vs 175 us at N = 128, 256 x 256).
+// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner). N does not enter: with
+// half an input image per CU and the output images filling the grid twice the two paths are within a few percent of each
+// other (bs = 8, K = 16, 256 x 256: 85 vs 91 us at N = 64, 144 vs 140 us at N = 128).
 int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
+    (void)N;
     if (algo != TURBOFNO_2D_AUTO) return algo;
     if (DX > 256 || DY > 256) return TURBOFNO_2D_THREE_KERNEL;      // an image no longer fits one block's LDS
-    const long in_images = (long)K * bs, out_images = (long)N * bs;
+    const long in_images = (long)K * bs;
     const bool big = DX == 256 && DY == 256;
-    const bool enough = in_images >= 256 || (in_images >= 128 && out_images >= 512);
+    const bool enough = in_images >= 256;
     return (enough && (big || bs >= 8)) ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
 }
 
@@ -267,7 +268,7 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
     float2* t1 = (float2*)ws;
     float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));
     if (int rc = hip_status(tfno::launch_fft_stride(logDX, (const float2*)x, t1, DY, (long)K * bs, st), "fft_stride launch")) return rc;
-    if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, algo_1d(), st), "fused_fft_cgemm_ifft launch")) return rc;
+    if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDY, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, algo_1d(), st, /*y_is_reread=*/true), "fused_fft_cgemm_ifft launch")) return rc;
     return hip_status(tfno::launch_ifft_stride(logDX, t2, (float2*)y, DY, (long)N * bs, st), "ifft_stride launch");
 }
 

@@ -56,7 +56,7 @@ inline hipError_t allow_dynamic_lds(const void* kernel, size_t bytes, std::atomi
 // 1D fused layer / Y stage of the three-kernel 2D pipeline. S = number of signals per channel.
 // algo: 0 = chosen by size, 1 = SIMT contraction, 2 / 3 = contraction on the matrix cores (512- / 256-thread blocks).
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
-                                       float2 alpha, int algo, hipStream_t stream);
+                                       float2 alpha, int algo, hipStream_t stream, bool y_is_reread = false);
 
 // Cluster variant of the fused 1D layer (layer1d_cluster.hip): cluster size for a problem (0 = not applicable), the
 // launch (hipErrorNotReady when its exchange buffer cannot be provided), and the bound of its inter-block waits in
@@ -69,7 +69,7 @@ void set_cluster_wait_ticks(unsigned long long ticks);
 // Large grids, DY = 128 / 256 (layer1d_wide.hip): one block per (signal set, 128 or 64 output channels), three-real-product
 // contraction.
 hipError_t launch_fused_wide(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
-                             hipStream_t stream);
+                             hipStream_t stream, int keep_y = 0);
 
 // Halves of the fused kernel (variants B and C) and the stand-alone contiguous transforms (variant A).
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

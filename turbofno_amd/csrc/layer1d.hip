@@ -20,7 +20,7 @@ namespace tfno {
 //           the column-major matrix A[m + k*M] (variant C).
 // FUSE_INV: the product goes straight into zero-padded backward transforms (variants C and D); otherwise it is
 //           stored as C[m + n*M] = alpha*A*W + beta*C (variant B).
-template <int LOGDY, bool FUSE_FWD, bool FUSE_INV>
+template <int LOGDY, bool FUSE_FWD, bool FUSE_INV, bool KEEP = false>
 __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                    const float2* __restrict__ W, float2* __restrict__ y,
                                                                    float2 alpha, float2 beta)
@@ -122,13 +122,11 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
             if constexpr (PAIR) {
                 pair128_backward(c, tw, exch, t16, yv);
                 float2* dst = y + ((long)(n0 + gpair + GROUPS * j) * S + s) * DY + t16;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
+                store_pair16<KEEP>(dst, (long)S * DY, yv);
             } else {
                 group_backward<LOGDY>(c, tw, exch, t, yv);
                 float2* dst = y + ((long)n * S + s) * DY + t;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) store_streaming(dst + L * i, yv[i]);
+                store_row16<L, KEEP>(dst, yv);
             }
         } else {
             float2* dst = y + s * 64 + t + (long)n * M;          // C[m + n*M], m = s*64 + t + L*i
@@ -181,7 +179,7 @@ template <int LOGDY, int THREADS_, int NT_ = 64> struct GeoMfma1D {
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(REGION0 + REGION1 + TWTAB);
 };
 
-template <int LOGDY, int THREADS, int NT>
+template <int LOGDY, int THREADS, int NT, bool KEEP = false>
 __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) void fused_fft_mfma_ifft_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                       const float2* __restrict__ W, float2* __restrict__ y,
                                                                       float2 alpha)
@@ -321,14 +319,12 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
         if constexpr (PAIR) {
             pair128_backward(c[pass], tw, exch, t16, yv);
             float2* dst = y + ((long)(n0 + gpair + KC * pass) * S + s) * DY + t16;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
+            store_pair16<KEEP>(dst, (long)S * DY, yv);
         } else {
             if constexpr (G::COMPACT) group_backward_lds<LOGDY>(c[pass], twrow, exch, t, yv);
             else group_backward<LOGDY>(c[pass], tw, exch, t, yv);
             float2* dst = y + ((long)(n0 + n) * S + s) * DY + t;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + L * i, yv[i]);
+            store_row16<L, KEEP>(dst, yv);
         }
     }
 }
@@ -356,7 +352,7 @@ TFNO_DEV float rotate8(float v)        // value of lane t ^ 8 of the same 16-lan
 }
 TFNO_DEV cpx rotate8(cpx v) { return make_float2(rotate8(v.x), rotate8(v.y)); }
 
-template <int LOGDY>
+template <int LOGDY, bool KEEP = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fused_fft_mfma_ifft_wave_kernel(
     int S, int N, int K, const float2* __restrict__ x, const float2* __restrict__ W, float2* __restrict__ y, float2 alpha)
 {
@@ -480,10 +476,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             for (int r = 0; r < 16; ++r) { e0[r] = exch[t * 17 + r]; e1[r] = exch1[t * 17 + r]; }
             inv_pass2_lds(e0, twrow, y0);
             inv_pass2_lds(e1, twrow, y1);
-#pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, y0[i]);
-#pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + (long)S * DY + 16 * i, y1[i]);
+            store_row16<16, KEEP>(dst, y0);
+            store_row16<16, KEEP>(dst + (long)S * DY, y1);
         } else {
             // lane t = r + 8 h finishes channel h: modes r + 8 c; even c come from lanes t < 8, odd c from lanes t >= 8
             cpx c8[8];
@@ -494,11 +488,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 c8[2 * a + 1] = upper ? c1[a] : got;
             }
             rows128_backward(c8, twrow, exch, t, y0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                store_streaming(dst + 16 * i, y0[i]);
-                store_streaming(dst + (long)S * DY + 16 * i, y0[8 + i]);
-            }
+            store_pair16<KEEP>(dst, (long)S * DY, y0);
         }
     }
 }
@@ -674,61 +664,84 @@ __global__ __launch_bounds__(256) void stride_DY_kernel(const float2* __restrict
     }
 }
 
-template <int LOGDY, bool FUSE_FWD, bool FUSE_INV>
-static hipError_t launch_fused_1d(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
-                                  float2 beta, hipStream_t stream)
+template <int LOGDY, bool FUSE_FWD, bool FUSE_INV, bool KEEP>
+static hipError_t launch_fused_1d_k(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                    float2 beta, hipStream_t stream)
 {
     using G = Geo1D<LOGDY>;
     if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
     if constexpr (G::LDS_BYTES > 64 * 1024) {          // DY = 128: 32 channels per chunk, 70 KiB
         static std::atomic<unsigned long long> served;
-        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV>),
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV, KEEP>),
                                              G::LDS_BYTES, served);
             e != hipSuccess)
             return e;
     }
     dim3 grid((unsigned)(S * (N / 64)), 1, 1), block(256, 1, 1);
-    hipLaunchKernelGGL((fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV>), grid, block, G::LDS_BYTES, stream, (int)S,
+    hipLaunchKernelGGL((fused_fft_cgemm_ifft_kernel<LOGDY, FUSE_FWD, FUSE_INV, KEEP>), grid, block, G::LDS_BYTES, stream, (int)S,
                        N, K, x, W, y, alpha, beta);
     return hipGetLastError();
 }
 
+// keep_y: the output is read again at once (Y stage of the three-kernel 2D pipeline): plain instead of streaming stores,
+// as a template parameter of the kernels - a run-time branch around the stores cost the 1D layer up to 20 %
+template <int LOGDY, bool FUSE_FWD, bool FUSE_INV>
+static hipError_t launch_fused_1d(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                  float2 beta, hipStream_t stream, int keep_y = 0)
+{
+    if constexpr (FUSE_FWD && FUSE_INV) {
+        if (keep_y) return launch_fused_1d_k<LOGDY, FUSE_FWD, FUSE_INV, true>(S, N, K, x, W, y, alpha, beta, stream);
+    }
+    return launch_fused_1d_k<LOGDY, FUSE_FWD, FUSE_INV, false>(S, N, K, x, W, y, alpha, beta, stream);
+}
+
 template <bool FUSE_FWD, bool FUSE_INV>
 static hipError_t dispatch_fused_1d(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
-                                    float2 alpha, float2 beta, hipStream_t stream)
+                                    float2 alpha, float2 beta, hipStream_t stream, int keep_y = 0)
 {
     switch (logDY) {
-    case 7: return launch_fused_1d<7, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
-    case 8: return launch_fused_1d<8, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
-    case 9: return launch_fused_1d<9, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
-    case 10: return launch_fused_1d<10, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream);
+    case 7: return launch_fused_1d<7, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream, keep_y);
+    case 8: return launch_fused_1d<8, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream, keep_y);
+    case 9: return launch_fused_1d<9, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream, keep_y);
+    case 10: return launch_fused_1d<10, FUSE_FWD, FUSE_INV>(S, N, K, x, W, y, alpha, beta, stream, keep_y);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <int LOGDY, int THREADS, int NT = 64>
-static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
-                                    hipStream_t stream)
+template <int LOGDY, int THREADS, int NT, bool KEEP>
+static hipError_t launch_fused_mfma_k(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                      hipStream_t stream)
 {
     using G = GeoMfma1D<LOGDY, THREADS, NT>;
     static std::atomic<unsigned long long> served;
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT>),
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT, KEEP>),
                                          G::LDS_BYTES, served);
         e != hipSuccess)
         return e;
     if (S * (N / NT) > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT>), dim3((unsigned)(S * (N / NT))), dim3(THREADS),
+    hipLaunchKernelGGL((fused_fft_mfma_ifft_kernel<LOGDY, THREADS, NT, KEEP>), dim3((unsigned)(S * (N / NT))), dim3(THREADS),
                        G::LDS_BYTES, stream, (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();
+}
+template <int LOGDY, int THREADS, int NT = 64>
+static hipError_t launch_fused_mfma(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
+                                    hipStream_t stream, int keep_y = 0)
+{
+    return keep_y ? launch_fused_mfma_k<LOGDY, THREADS, NT, true>(S, N, K, x, W, y, alpha, stream)
+                  : launch_fused_mfma_k<LOGDY, THREADS, NT, false>(S, N, K, x, W, y, alpha, stream);
 }
 
 template <int LOGDY>
 static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
-                                    hipStream_t stream)
+                                    hipStream_t stream, int keep_y = 0)
 {
     if (S * (N / 64) > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(fused_fft_mfma_ifft_wave_kernel<LOGDY>, dim3((unsigned)(S * (N / 64))), dim3(64), 0, stream, (int)S, N, K,
-                       x, W, y, alpha);
+    if (keep_y)
+        hipLaunchKernelGGL((fused_fft_mfma_ifft_wave_kernel<LOGDY, true>), dim3((unsigned)(S * (N / 64))), dim3(64), 0, stream, (int)S, N,
+                           K, x, W, y, alpha);
+    else
+        hipLaunchKernelGGL((fused_fft_mfma_ifft_wave_kernel<LOGDY, false>), dim3((unsigned)(S * (N / 64))), dim3(64), 0, stream, (int)S,
+                           N, K, x, W, y, alpha);
     return hipGetLastError();
 }
 
@@ -738,8 +751,11 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
 // 7 = matrix cores, a cluster of blocks splits the K channels of one signal set (DY = 256, N = 64 / 128, small grids),
 // 8 = matrix cores, 256-thread blocks with tiles of 128 output channels, three real products per complex one (DY = 256)
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
-                                       float2 alpha, int algo, hipStream_t stream)
+                                       float2 alpha, int algo, hipStream_t stream, bool y_is_reread)
 {
+    // y_is_reread (Y stage of the three-kernel 2D pipeline): the block kernels and the SIMT kernel then leave y in the
+    // caches instead of streaming it past them; the other kernels ignore it
+    const int keep_y = y_is_reread ? 1 : 0;
     // by size (measured on MI355X):
     //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
     //    every K, even K = 8 where most of a chunk is padding;
@@ -755,27 +771,27 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     const bool built = logDY >= 7 && logDY <= 10;
     const bool long_signal = logDY >= 9;            // 512 / 1024: on large grids the block kernels tie with the SIMT kernel
     const long items = S * (N / 64);
-    if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
-    if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
+    if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
     // N a multiple of 128, DY = 256, K >= 16: blocks with tiles of 128 output channels (every input channel transformed
     // once per signal set, three real products per complex one): 5-20 % ahead of the kernels below on every grid that
     // fills its two slots per CU reasonably evenly (measured from 400 blocks up; with a last round under three quarters
     // full the 64-channel kernels, with their finer blocks, are ahead)
     if (algo == 0 && logDY == 8 && N % 128 == 0 && K >= 16) {
         const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
-        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream);
+        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream, keep_y);
     }
     // the same at DY = 128 for K >= 64 (3-21 % ahead up to 64 blocks per CU; with fewer channels, or on the very largest
     // grids, the one-wavefront kernel below is level or ahead)
     if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 64) {
         const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
         if (blocks > cu_count() && blocks <= 64L * cu_count() && 4 * blocks >= 3 * rounds * slots)
-            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream);
+            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
     }
     if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
-        return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream);
+        return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
     if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cu_count() : (K >= 24 && items >= 128L * cu_count())))
-        return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream);
+        return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream, keep_y);
     // small grids, 64 channels or more, N = 64 / 128: a cluster of blocks per signal set, no forward transform twice.
     // Without its exchange buffer (first use inside a stream capture, out of memory) the kernels below take over.
     if (algo == 7 || (algo == 0 && logDY == 8 && K >= 64)) {
@@ -786,7 +802,7 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         }
         if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
     }
-    if (algo == 8 && (logDY == 7 || logDY == 8)) return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream);
+    if (algo == 8 && (logDY == 7 || logDY == 8)) return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream, keep_y);
     if (algo == 8) algo = 0;
     int pick = algo == 4 ? 2 : algo;
     if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (!long_signal ? 3 : 1);
@@ -804,18 +820,18 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     }
     // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
     if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
-        return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream);
+        return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
     if (pick == 2 && logDY == 7 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
-        return launch_fused_mfma<7, 512, 32>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 3 && logDY == 9) return launch_fused_mfma<9, 256>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 3 && logDY == 10) return launch_fused_mfma<10, 256>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 2 && logDY == 9) return launch_fused_mfma<9, 512>(S, N, K, x, W, y, alpha, stream);
-    if (pick == 2 && logDY == 10) return launch_fused_mfma<10, 512>(S, N, K, x, W, y, alpha, stream);
-    return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream);
+        return launch_fused_mfma<7, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 3 && logDY == 9) return launch_fused_mfma<9, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 3 && logDY == 10) return launch_fused_mfma<10, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 2 && logDY == 9) return launch_fused_mfma<9, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+    if (pick == 2 && logDY == 10) return launch_fused_mfma<10, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+    return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream, keep_y);
 }
 
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

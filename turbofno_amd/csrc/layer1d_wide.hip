@@ -33,7 +33,7 @@ template <int NT> struct GeoWide {
     static_assert(WROW % 64 == 16, "rows of an operand fetch must be 16 banks apart");
 };
 
-template <int NT>
+template <int NT, bool KEEP>
 __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                          const float2* __restrict__ W, float2* __restrict__ y,
                                                                          float2 alpha)
@@ -142,8 +142,7 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide_kernel(int S,
         for (int a = 0; a < 4; ++a) c[a] = buf[g * PC + t + 16 * a];
         group_backward<8>(c, tw, exch, t, yv);
         float2* dst = y + ((long)(n0 + 16 * i + g) * S + s) * DY + t;
-#pragma unroll
-        for (int j = 0; j < 16; ++j) store_streaming(dst + 16 * j, yv[j]);
+        store_row16<16, KEEP>(dst, yv);
     }
 }
 
@@ -151,7 +150,7 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide_kernel(int S,
 // round of the block covers 32 channels: the spectra tile holds 32 channels, the W'' tile 16 - it is built and multiplied
 // twice per round, and the rows of W for the second half are fetched while the first half is being multiplied. The
 // product goes to LDS 32 channels at a time.
-template <int NT>
+template <int NT, bool KEEP>
 __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide128_kernel(int S, int N, int K, const float2* __restrict__ x,
                                                                             const float2* __restrict__ W, float2* __restrict__ y,
                                                                             float2 alpha)
@@ -276,12 +275,11 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide128_kernel(int
         __syncthreads();                                        // the buffer is consumed: the next step may overwrite it
         pair128_backward(c, tw, exch, t16, yv);
         float2* dst = y + ((long)(n0 + 32 * step + 2 * grp) * S + s) * DY + t16;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { store_streaming(dst + 16 * i, yv[i]); store_streaming(dst + (long)S * DY + 16 * i, yv[8 + i]); }
+        store_pair16<KEEP>(dst, (long)S * DY, yv);
     }
 }
 
-template <int NT>
+template <int NT, bool KEEP>
 static hipError_t launch_wide_t(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
                                 hipStream_t stream)
 {
@@ -289,21 +287,23 @@ static hipError_t launch_wide_t(int logDY, long S, int N, int K, const float2* x
     if (S * (N / NT) > 0x7fffffffL) return hipErrorInvalidValue;
     static_assert(G::LDS_BYTES <= 64 * 1024, "no attribute call needed below 64 KiB of dynamic LDS");
     if (logDY == 7)
-        hipLaunchKernelGGL(fused_fft_mfma_ifft_wide128_kernel<NT>, dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream,
+        hipLaunchKernelGGL((fused_fft_mfma_ifft_wide128_kernel<NT, KEEP>), dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream,
                            (int)S, N, K, x, W, y, alpha);
     else
-        hipLaunchKernelGGL(fused_fft_mfma_ifft_wide_kernel<NT>, dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream, (int)S,
-                           N, K, x, W, y, alpha);
+        hipLaunchKernelGGL((fused_fft_mfma_ifft_wide_kernel<NT, KEEP>), dim3((unsigned)(S * (N / NT))), dim3(256), G::LDS_BYTES, stream,
+                           (int)S, N, K, x, W, y, alpha);
     return hipGetLastError();
 }
 
 // DY = 128 or 256. Tiles of 128 output channels when N allows, else of 64.
 hipError_t launch_fused_wide(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y, float2 alpha,
-                             hipStream_t stream)
+                             hipStream_t stream, int keep_y)
 {
     if (logDY != 7 && logDY != 8) return hipErrorInvalidValue;
-    if (N % 128 == 0) return launch_wide_t<128>(logDY, S, N, K, x, W, y, alpha, stream);
-    return launch_wide_t<64>(logDY, S, N, K, x, W, y, alpha, stream);
+    // keep_y: plain instead of streaming stores of y, for a consumer that reads it at once (a template parameter of the kernels)
+    if (N % 128 == 0)
+        return keep_y ? launch_wide_t<128, true>(logDY, S, N, K, x, W, y, alpha, stream) : launch_wide_t<128, false>(logDY, S, N, K, x, W, y, alpha, stream);
+    return keep_y ? launch_wide_t<64, true>(logDY, S, N, K, x, W, y, alpha, stream) : launch_wide_t<64, false>(logDY, S, N, K, x, W, y, alpha, stream);
 }
 
 }  // namespace tfno

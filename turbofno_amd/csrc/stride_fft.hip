@@ -143,6 +143,94 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
     for (int i = 0; i < 16; ++i) store_streaming(dst + (long)L * i * DY, yv[i]);
 }
 
+// Backward kernel of lengths 512 / 1024, persistent: a block walks panels blockIdx.x, + gridDim.x, ... and fetches the retained rows of
+// its next panel (2 to 8 values per thread) as soon as those of the current one are in LDS. Inside the three-kernel
+// pipeline these rows come from HBM while the memory system is saturated with this kernel's own stores; without the
+// look-ahead every block began with that exposed latency (length 512, 1024 images: 587 us in the pipeline against 416 us
+// with the input resident in the Infinity Cache).
+template <int LOGDX, int COLS>
+__global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride_persistent_kernel(const float2* __restrict__ in,
+                                                                                     float2* __restrict__ out, int DY, long npanels)
+{
+    using G = GeoStride<LOGDX, COLS>;
+    constexpr int DX = G::DX, L = G::L;
+    static_assert(LOGDX >= 9, "lengths up to 256 use ifft_stride_kernel");
+    constexpr int NIN = 64 / L < 4 ? (L == 8 ? 8 : 4) : 64 / L;   // retained rows per thread: 2 / 1 (L = 32 / 64), 4 (16), 8 (8)
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, yl = tid % COLS, t = tid / COLS;
+
+    cpx tw[16];
+    load_lane_twiddles<LOGDX>(t, tw);
+    // rows of the retained block a thread reads, in the order its first step wants them
+    auto fetch = [&](cpx (&c)[NIN], long panel) {
+        const long col = panel * COLS + yl;
+        const float2* src = in + (col / DY) * 64 * DY + (int)(col % DY);
+        if constexpr (L >= 32) {
+#pragma unroll
+            for (int mm = 0; mm < 64 / L; ++mm) c[mm] = src[(long)(t + L * mm) * DY];
+        } else if constexpr (L == 16) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) c[s] = src[(long)(t + 16 * s) * DY];
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) { c[s] = src[(long)(t + 16 * s) * DY]; c[4 + s] = src[(long)(t + 8 + 16 * s) * DY]; }
+        }
+    };
+    cpx c[NIN];
+    long panel = blockIdx.x;
+    if (panel < npanels) fetch(c, panel);
+    for (; panel < npanels; panel += gridDim.x) {
+        const long col = panel * COLS + yl;
+        const long sig = col / DY;
+        const int y = (int)(col % DY);
+        if constexpr (L >= 32) {
+#pragma unroll
+            for (int mm = 0; mm < 64 / L; ++mm) lds[(t + L * mm) * COLS + yl] = c[mm];
+        } else if constexpr (L == 16) {
+            cpx c4[4], h[16];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) c4[s] = c[s];
+            dft16_pad4<+1>(c4, h);
+#pragma unroll
+            for (int tt = 0; tt < 16; ++tt) lds[(tt * 17 + t) * COLS + yl] = h[tt];
+        } else {
+            cpx c0[4], c1[4], h0[8], h1[8];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) { c0[s] = c[s]; c1[s] = c[4 + s]; }
+            dft8_pad4<+1>(c0, h0);
+            dft8_pad4<+1>(c1, h1);
+#pragma unroll
+            for (int tt = 0; tt < 8; ++tt) {
+                lds[(tt * 17 + t) * COLS + yl] = h0[tt];
+                lds[(tt * 17 + t + 8) * COLS + yl] = h1[tt];
+            }
+        }
+        if (panel + gridDim.x < npanels) fetch(c, panel + gridDim.x);      // look-ahead: travels under the rest of this panel
+        __syncthreads();
+        cpx e[16], yv[16];
+        if constexpr (L >= 32) {
+            // first-pass inputs from the 64 retained rows: twiddle once per four row groups, 4-point transform, second small
+            // exchange (wide_backward_partial / wide_back_index on this kernel's [.][yl] layout)
+            cpx part[16];
+            wide_backward_partial<L>(lds + yl, COLS, t, part);
+            __syncthreads();                                 // every thread has read the 64 rows
+#pragma unroll
+            for (int k = 0; k < 16; ++k) lds[wide_back_index<L>(t, k) * COLS + yl] = part[k];
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * COLS + yl];
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) e[r] = lds[(t * 17 + r) * COLS + yl];
+        }
+        inv_pass2(e, tw, yv);
+        float2* dst = out + (sig * DX + t) * DY + y;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) store_streaming(dst + (long)L * i * DY, yv[i]);
+        __syncthreads();                                     // the exchange array is free for the next panel
+    }
+}
+
 template <int LOGDX, bool INVERSE, int COLS>
 static hipError_t launch_stride_c(const float2* in, float2* out, int DY, long nsig, hipStream_t stream)
 {
@@ -155,6 +243,27 @@ static hipError_t launch_stride_c(const float2* in, float2* out, int DY, long ns
         const void* fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX, COLS>)
                                  : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX, COLS>);
         if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served); e != hipSuccess) return e;
+    }
+    if constexpr (INVERSE && LOGDX >= 9) {
+        // persistent grid: as many blocks as are resident at once. Lengths up to 256 keep one block per panel: their
+        // input (at most 128 MiB at bs = 16) is still in the caches when the kernel runs, and the persistent form was
+        // measured 3-8 % slower there.
+        static std::atomic<int> per_cu[64];
+        int dev = 0;
+        if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+        int occ = per_cu[dev & 63].load(std::memory_order_relaxed);
+        if (occ <= 0) {
+            if (hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ifft_stride_persistent_kernel<LOGDX, COLS>, G::THREADS,
+                                                                            G::LDS_BYTES);
+                e != hipSuccess)
+                return e;
+            if (occ <= 0) occ = 1;
+            per_cu[dev & 63].store(occ, std::memory_order_relaxed);
+        }
+        const long resident = (long)occ * cu_count();
+        hipLaunchKernelGGL((ifft_stride_persistent_kernel<LOGDX, COLS>), dim3((unsigned)(blocks < resident ? blocks : resident)), block,
+                           G::LDS_BYTES, stream, in, out, DY, blocks);
+        return hipGetLastError();
     }
     if (INVERSE) hipLaunchKernelGGL((ifft_stride_kernel<LOGDX, COLS>), grid, block, G::LDS_BYTES, stream, in, out, DY);
     else hipLaunchKernelGGL((fft_stride_kernel<LOGDX, COLS>), grid, block, G::LDS_BYTES, stream, in, out, DY);
