@@ -80,6 +80,51 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void fft_stride_
     }
 }
 
+// Forward kernel of lengths 512 / 1024, persistent: a block walks panels blockIdx.x, + gridDim.x, ... and issues the loads
+// of its next panel as soon as the first pass has consumed the registers of the current one. At these lengths only one or
+// two blocks fit a CU (the exchange array), so without the look-ahead the memory system idles while a block computes.
+template <int LOGDX, int COLS>
+__global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void fft_stride_persistent_kernel(const float2* __restrict__ in,
+                                                                                               float2* __restrict__ out, int DY,
+                                                                                               long npanels)
+{
+    using G = GeoStride<LOGDX, COLS>;
+    constexpr int DX = G::DX, L = G::L;
+    static_assert(LOGDX >= 9, "lengths up to 256 use fft_stride_kernel");
+    extern __shared__ float2 lds[];
+    const int tid = threadIdx.x, yl = tid % COLS, t = tid / COLS;
+    cpx tw[16], v[16];
+    load_lane_twiddles<LOGDX>(t, tw);
+    auto fetch = [&](long panel) {
+        const long col = panel * COLS + yl;
+        const float2* src = in + ((col / DY) * DX + t) * DY + (int)(col % DY);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = src[(long)L * i * DY];
+    };
+    long panel = blockIdx.x;
+    if (panel < npanels) fetch(panel);
+    for (; panel < npanels; panel += gridDim.x) {
+        const long col = panel * COLS + yl;
+        float2* dst = out + (col / DY) * 64 * DY + (int)(col % DY);
+        cpx g[16];
+        fwd_pass1(v, tw, g);
+        if (panel + gridDim.x < npanels) fetch(panel + gridDim.x);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lds[(t * 17 + r) * COLS + yl] = g[r];
+        __syncthreads();
+        cpx inner[4], o[64 / L];
+        wide_forward_inner<L>(lds + yl, COLS, t, inner);
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 4; ++c) lds[wide_swap_index<L>(t / (L / 16), c, t % (L / 16)) * COLS + yl] = inner[c];
+        __syncthreads();
+        wide_forward_outer<L>(lds + yl, COLS, t, o);
+#pragma unroll
+        for (int mm = 0; mm < 64 / L; ++mm) dst[(long)wide_mode<L>(t, mm) * DY] = o[mm];
+        __syncthreads();                                     // the exchange array is free for the next panel
+    }
+}
+
 template <int LOGDX, int COLS>
 __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride_kernel(const float2* __restrict__ in,
                                                                                      float2* __restrict__ out, int DY)
@@ -240,11 +285,17 @@ static hipError_t launch_stride_c(const float2* in, float2* out, int DY, long ns
     dim3 grid((unsigned)blocks, 1, 1), block(G::THREADS, 1, 1);
     if constexpr (G::LDS_BYTES > 64 * 1024) {
         static std::atomic<unsigned long long> served;
-        const void* fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX, COLS>)
-                                 : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX, COLS>);
+        const void* fn;                                  // the kernel that is launched below
+        if constexpr (INVERSE ? LOGDX >= 9 : LOGDX >= 10)
+            fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_persistent_kernel<LOGDX, COLS>)
+                         : reinterpret_cast<const void*>(fft_stride_persistent_kernel<LOGDX, COLS>);
+        else
+            fn = INVERSE ? reinterpret_cast<const void*>(ifft_stride_kernel<LOGDX, COLS>)
+                         : reinterpret_cast<const void*>(fft_stride_kernel<LOGDX, COLS>);
         if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served); e != hipSuccess) return e;
     }
-    if constexpr (INVERSE && LOGDX >= 9) {
+    constexpr bool PERSISTENT = INVERSE ? LOGDX >= 9 : LOGDX >= 10;   // forward, length 512: no gain measured
+    if constexpr (PERSISTENT) {
         // persistent grid: as many blocks as are resident at once. Lengths up to 256 keep one block per panel: their
         // input (at most 128 MiB at bs = 16) is still in the caches when the kernel runs, and the persistent form was
         // measured 3-8 % slower there.
@@ -253,16 +304,18 @@ static hipError_t launch_stride_c(const float2* in, float2* out, int DY, long ns
         if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
         int occ = per_cu[dev & 63].load(std::memory_order_relaxed);
         if (occ <= 0) {
-            if (hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ifft_stride_persistent_kernel<LOGDX, COLS>, G::THREADS,
-                                                                            G::LDS_BYTES);
-                e != hipSuccess)
-                return e;
+            const hipError_t e = INVERSE ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, ifft_stride_persistent_kernel<LOGDX, COLS>,
+                                                                                        G::THREADS, G::LDS_BYTES)
+                                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fft_stride_persistent_kernel<LOGDX, COLS>,
+                                                                                        G::THREADS, G::LDS_BYTES);
+            if (e != hipSuccess) return e;
             if (occ <= 0) occ = 1;
             per_cu[dev & 63].store(occ, std::memory_order_relaxed);
         }
         const long resident = (long)occ * cu_count();
-        hipLaunchKernelGGL((ifft_stride_persistent_kernel<LOGDX, COLS>), dim3((unsigned)(blocks < resident ? blocks : resident)), block,
-                           G::LDS_BYTES, stream, in, out, DY, blocks);
+        const dim3 pgrid((unsigned)(blocks < resident ? blocks : resident));
+        if (INVERSE) hipLaunchKernelGGL((ifft_stride_persistent_kernel<LOGDX, COLS>), pgrid, block, G::LDS_BYTES, stream, in, out, DY, blocks);
+        else hipLaunchKernelGGL((fft_stride_persistent_kernel<LOGDX, COLS>), pgrid, block, G::LDS_BYTES, stream, in, out, DY, blocks);
         return hipGetLastError();
     }
     if (INVERSE) hipLaunchKernelGGL((ifft_stride_kernel<LOGDX, COLS>), grid, block, G::LDS_BYTES, stream, in, out, DY);
