@@ -28,7 +28,7 @@ def check(got, ref, tol, what):
 
 # S, K, N -> cluster size / channels per member / chunk (on 256 CUs)
 SHAPES = [
-    (64, 128, 128),   # BASELINE large-hidden case: 4 members x 32 channels, one chunk of 32
+    (64, 128, 128),   # the large-hidden benchmark case: 4 members x 32 channels, one chunk of 32
     (64, 64, 128),    # 4 x 16, chunk 16
     (32, 128, 128),   # 8 members x 16 channels, 16 output channels each
     (13, 64, 128),    # S not a multiple of 8: padding blocks of the last group of clusters leave at once
