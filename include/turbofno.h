@@ -41,6 +41,7 @@ extern "C" {
 #define TURBOFNO_2D_AUTO          0
 #define TURBOFNO_2D_THREE_KERNEL  1  /* X transform, fused Y stage, X inverse: the reference's structure */
 #define TURBOFNO_2D_WHOLE_IMAGE   2  /* one block per image + matrix-core CGEMM                          */
+#define TURBOFNO_2D_ROWS_FIRST    3  /* Y transform of whole rows, fused X stage, Y inverse of whole rows */
 
 /*
  * Fused 1D layer kernel. Replaces the table entries fused_fft_cgemm_ifft[log2(DY)-7]
@@ -84,7 +85,9 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
  * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE once K*bs images fill the CUs, THREE_KERNEL below; the workspace query
- * with the same arguments makes the same choice.
+ * with the same arguments makes the same choice. ROWS_FIRST is the three-stage structure with the axes exchanged
+ * (the contiguous axis is transformed first and last, so that x and y move as whole rows): same result, the 2D
+ * transform being separable; its intermediates are [images][64][DX].
  */
 size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, int algo);
 int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const void* W, void* y,

@@ -93,7 +93,7 @@ def _check_batch_slices(y, x_h, W_h, alpha, batch_elements, tol, what):
         assert e2 <= tol["l2"] and em <= tol["max"] and ee <= tol["elem"], (what, b, e2, em, ee)
 
 
-@pytest.mark.parametrize("algo", [0, 1, 2])
+@pytest.mark.parametrize("algo", [0, 1, 2, 3])
 def test_headline_against_oracle_slices(algo, tol):
     """configuration 5 (bs=16, 256 x 256, K=N=64, Gaussian random field) at full size; batch elements 0, 7, 15
     against the oracle"""
@@ -110,11 +110,28 @@ def test_config4_bs16_against_oracle_slices(D, K, tol):
     """configuration 4 at its largest batch, every algorithm, batch elements 0, 5, 15 against the oracle"""
     x_h, W_h = workloads.uniform_2d(440 + D + K, 16, D, D, K, 64)
     x, W = torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
-    for algo in (0, 1, 2):
+    for algo in (0, 1, 2, 3):
         print("config4 bs=16 vs oracle slices", D, K, "algo", algo, flush=True)
         y = tf.layer_2d(x, W, alpha=1 - 1j, algo=algo)
         torch.cuda.synchronize()
         _check_batch_slices(y, x_h, W_h, 1 - 1j, (0, 5, 15), tol, "config4 D=%d K=%d algo %d" % (D, K, algo))
+
+
+@pytest.mark.parametrize("bs,DX,DY,K,N,algo", [
+    (4, 512, 512, 32, 64, 0),        # whole rows first by size: 2048 row blocks of 32 rows on at most 768 persistent blocks
+    (4, 256, 1024, 32, 64, 0),       # DY > DX: whole rows first, row blocks of 16 rows
+    (4, 1024, 256, 32, 64, 0),       # DX > DY: X axis first
+    (6, 512, 512, 24, 128, 1),
+    (6, 512, 512, 24, 128, 3),
+])
+def test_large_images_against_oracle_slices(bs, DX, DY, K, N, algo, tol):
+    """lengths above 256 at sizes that run the persistent loops of the X-axis kernels and of the row kernels several times
+    per block; first and last batch element against the oracle"""
+    print("large images", bs, DX, DY, K, N, "algo", algo, flush=True)
+    x_h, W_h = workloads.uniform_2d(950 + bs + DX + K + algo, bs, DX, DY, K, N)
+    y = tf.layer_2d(torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda(), alpha=0.5 - 1j, algo=algo)
+    torch.cuda.synchronize()
+    _check_batch_slices(y, x_h, W_h, 0.5 - 1j, (0, bs - 1), tol, "large images %dx%d algo %d" % (DX, DY, algo))
 
 
 @pytest.mark.parametrize("bs,DX,DY,K,N", [

@@ -15,7 +15,7 @@ def _rel(a, b):
     return float(torch.linalg.vector_norm(a - b) / torch.linalg.vector_norm(b))
 
 
-@pytest.mark.parametrize("algo", [1, 2])
+@pytest.mark.parametrize("algo", [1, 2, 3])
 def test_layer_2d_in_a_graph(algo):
     print("graph 2d algo", algo, flush=True)
     bs, D, K, N = 4, 128, 64, 64

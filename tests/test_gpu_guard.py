@@ -37,7 +37,7 @@ def test_layer_1d_stays_in_bounds(bs, DY, K, N, algo, algo_1d):
     assert not bool((y == CANARY).any())            # and the output itself was written everywhere
 
 
-@pytest.mark.parametrize("algo", [1, 2])
+@pytest.mark.parametrize("algo", [1, 2, 3])
 @pytest.mark.parametrize("bs,DX,DY,K,N", [(3, 128, 256, 24, 64), (1, 256, 128, 72, 128), (5, 128, 128, 8, 64),
                                           (2, 256, 256, 40, 64)])
 def test_layer_2d_stays_in_bounds(bs, DX, DY, K, N, algo):

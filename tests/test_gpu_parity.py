@@ -133,9 +133,22 @@ def test_stride_stages(DX, DY, nsig, tol):
     (3, 128, 256, 8, 64, 2),
     (2, 256, 128, 24, 128, 2),
     (5, 128, 128, 8, 64, 0),         # auto: 40 input images, below the whole-image threshold -> three-kernel path
-    (1, 512, 128, 8, 64, 0),         # lengths above 256: auto = three-kernel path
+    (1, 512, 128, 8, 64, 0),         # lengths above 256, DX > DY: auto = three-kernel path (X axis first)
     (1, 256, 1024, 16, 64, 1),
     (2, 1024, 512, 8, 64, 0),
+    (1, 256, 1024, 16, 64, 0),       # DY > DX: auto = whole rows first
+    (1, 512, 512, 8, 64, 0),         # square, few images: X axis first
+    (2, 512, 512, 64, 64, 0),        # square, K * bs = 128: whole rows first
+    (1, 1024, 1024, 8, 64, 0),
+    (1, 128, 128, 16, 64, 3),        # whole rows first on every pair of lengths (row blocks of 32, 32, 32 and 16 rows)
+    (2, 256, 128, 8, 64, 3),
+    (3, 128, 256, 24, 128, 3),
+    (1, 256, 256, 72, 64, 3),
+    (1, 512, 256, 8, 64, 3),
+    (2, 128, 512, 16, 64, 3),
+    (1, 1024, 128, 8, 64, 3),
+    (1, 512, 1024, 8, 128, 3),
+    (5, 128, 128, 8, 64, 3),         # 20 row blocks of 32 rows over 40 images: several images per persistent block
 ])
 def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     print("case layer_2d", bs, DX, DY, K, N, algo, flush=True)
@@ -146,15 +159,15 @@ def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     check(y, oracle.layer_2d(x, W, alpha), tol, "layer_2d algo=%d" % algo)
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(16))
 def test_layer_2d_random_shapes(seed, tol):
-    """seeded random 2D shapes through the size rule, the three-kernel path and the whole-image path"""
+    """seeded random 2D shapes through the size rule, the three-kernel path, the whole-image path and whole rows first"""
     rng = np.random.default_rng(2000 + seed)
     DX, DY = int(rng.choice([128, 256])), int(rng.choice([128, 256]))
     K = 8 * int(rng.integers(1, 12))
     N = 64 * int(rng.integers(1, 3))
     bs = int(rng.integers(1, 4))
-    algo = seed % 3
+    algo = seed % 4
     alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
     print("case layer_2d random", seed, "bs", bs, DX, DY, "K", K, "N", N, "algo", algo, flush=True)
     x, W = workloads.uniform_2d(seed, bs, DX, DY, K, N)

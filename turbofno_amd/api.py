@@ -198,7 +198,8 @@ def _layer_2d_operands(x, W, y):
 
 def layer_2d(x, W, y=None, alpha=1.0 + 0j, workspace=None, algo=0):
     """x: [K][bs][DX][DY], W: [N][K] -> y: [N][bs][DX][DY]. `workspace`: uint8 GPU tensor (allocated
-    here when omitted; pass one to keep allocation out of a timed loop)."""
+    here when omitted; pass one to keep allocation out of a timed loop). algo: 0 by size, 1 three kernels with the X
+    axis first, 2 one block per image, 3 three kernels with whole rows first."""
     K, bs, DX, DY, N, y = _layer_2d_operands(x, W, y)
     need = layer_2d_workspace_bytes(bs, DX, DY, K, N, algo)
     if workspace is None:

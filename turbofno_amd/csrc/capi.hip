@@ -60,7 +60,13 @@ int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
     (void)N;
     if (algo != TURBOFNO_2D_AUTO) return algo;
-    if (DX > 256 || DY > 256) return TURBOFNO_2D_THREE_KERNEL;      // an image no longer fits one block's LDS
+    if (DX > 256 || DY > 256) {
+        // an image no longer fits one block's LDS: three stages. The axis that is transformed first is the one whose
+        // truncation shrinks the intermediates most, i.e. the longer one (DY = 4 DX: half the time of the other order;
+        // DX = 4 DY: the reverse). Square images: whole rows first (9-18 % ahead) unless the grid is small.
+        if (DY != DX) return DY > DX ? TURBOFNO_2D_ROWS_FIRST : TURBOFNO_2D_THREE_KERNEL;
+        return (DY >= 1024 || (long)K * bs >= 128) ? TURBOFNO_2D_ROWS_FIRST : TURBOFNO_2D_THREE_KERNEL;
+    }
     const long in_images = (long)K * bs;
     const bool big = DX == 256 && DY == 256;
     const bool enough = in_images >= 256;
@@ -228,7 +234,8 @@ size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, i
     if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
     if (pick_algo(bs, DX, DY, K, N, algo) == TURBOFNO_2D_WHOLE_IMAGE)
         return align256((size_t)K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
-    return align256((size_t)K * bs * 64 * DY * sizeof(float2)) + align256((size_t)N * bs * 64 * DY * sizeof(float2));
+    const int kept_rows_of = pick_algo(bs, DX, DY, K, N, algo) == TURBOFNO_2D_ROWS_FIRST ? DX : DY;
+    return align256((size_t)K * bs * 64 * kept_rows_of * sizeof(float2)) + align256((size_t)N * bs * 64 * kept_rows_of * sizeof(float2));
 }
 
 // Both 2D entry points: validation, choice of algorithm, the three launches. `workspace` is the caller's buffer
@@ -246,7 +253,7 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
         return fail(TURBOFNO_ERR_INVALID_ARG, "K*bs=%ld or N*bs=%ld images exceed the grid limit", (long)K * bs, (long)N * bs);
     if (!length_built(logDX) || !length_built(logDY))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256, 512, 1024} are built", DX, DY);
-    if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE)
+    if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE && algo != TURBOFNO_2D_ROWS_FIRST)
         return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
     if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256))
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the whole-image path is built for lengths in {128, 256}", DX, DY);
@@ -264,6 +271,13 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
         if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, K * bs, st), "fft2d_trunc launch")) return rc;
         if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, make_float2(0.f, 0.f), st), "cgemm_modes launch")) return rc;
         return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, N * bs, st), "ifft2d_pad launch");
+    }
+    if (a == TURBOFNO_2D_ROWS_FIRST) {
+        float2* t1 = (float2*)ws;
+        float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DX * sizeof(float2)));
+        if (int rc = hip_status(tfno::launch_fft_rows_trunc(logDY, (const float2*)x, t1, DX, (long)K * bs, st), "fft_rows_trunc launch")) return rc;
+        if (int rc = hip_status(tfno::launch_fused_fft_cgemm_ifft(logDX, (long)bs * 64, N, K, t1, (const float2*)W, t2, alpha, algo_1d(), st, /*y_is_reread=*/true), "fused_fft_cgemm_ifft launch")) return rc;
+        return hip_status(tfno::launch_ifft_rows_pad(logDY, t2, (float2*)y, DX, (long)N * bs, st), "ifft_rows_pad launch");
     }
     float2* t1 = (float2*)ws;
     float2* t2 = (float2*)(ws + align256((size_t)K * bs * 64 * DY * sizeof(float2)));

@@ -83,6 +83,11 @@ hipError_t launch_ifft_stride_DY(int logDY, const float2* in, float2* out, long 
 hipError_t launch_fft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream);
 hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, long nsig, hipStream_t stream);
 
+// Y-axis (contiguous) transforms of the rows-first 2D pipeline (rows_fft.hip): in[img][DX][DY] -> out[img][64][DX] and
+// back; the intermediates are transposed so that the fused 1D kernel runs along X on them.
+hipError_t launch_fft_rows_trunc(int logDY, const float2* in, float2* out, int DX, long nimg, hipStream_t stream);
+hipError_t launch_ifft_rows_pad(int logDY, const float2* in, float2* out, int DX, long nimg, hipStream_t stream);
+
 // Whole-image 2D path (DX, DY in {128, 256}): truncated 2D forward transform per image, mode-space CGEMM
 // on the matrix cores, zero-padded 2D backward transform per image. nimg: the C ABI rejects counts beyond INT_MAX.
 hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, int nimg, hipStream_t stream);
