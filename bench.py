@@ -23,7 +23,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--bs", type=int, default=16)
-    ap.add_argument("--algo", type=int, default=0, help="0 auto, 1 three-kernel pipeline, 2 whole-image")
+    ap.add_argument("--algo", type=int, default=0, help="0 auto, 1 three-kernel pipeline, 2 whole-image, 3 three kernels with whole rows first")
     ap.add_argument("--settle-ms", type=float, default=60.0,
                     help="untimed GPU activity (the same layer) before the warm-up steps: a fresh GPU needs ~20 ms of load "
                          "before its clocks settle, and the first steps after an idle period run ~8 %% slower")
@@ -214,7 +214,7 @@ def main():
         "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "complex64 (fp32 arithmetic)", "data": "synthetic",
         "config": {"workload": "2D layer bs=%d 256x256 K=64 N=64, 64x64 modes, Gaussian random field input" % bs,
-                   "algo": ("auto -> " if args.algo == 0 else "") + {1: "three-kernel", 2: "whole-image"}[algo]},
+                   "algo": ("auto -> " if args.algo == 0 else "") + {1: "three-kernel", 2: "whole-image", 3: "three-kernel, rows first"}[algo]},
         "settle": {"ms": args.settle_ms, "steps": settle_steps},
         "env": {"HIP_FORCE_DEV_KERNARG": os.environ.get("HIP_FORCE_DEV_KERNARG")},
         "layer_algorithmic_bytes": layer_bytes, "layer_GBps": round(layer_gbs, 1),
