@@ -119,7 +119,7 @@ def test_config4_bs16_against_oracle_slices(D, K, tol):
 
 @pytest.mark.parametrize("bs,DX,DY,K,N,algo", [
     (4, 512, 512, 32, 64, 0),        # whole rows first by size: 2048 row blocks of 32 rows on at most 768 persistent blocks
-    (4, 256, 1024, 32, 64, 0),       # DY > DX: whole rows first, row blocks of 16 rows
+    (4, 256, 1024, 32, 64, 0),       # DY > DX: whole rows first, eight batches of rows per block
     (4, 1024, 256, 32, 64, 0),       # DX > DY: X axis first
     (6, 512, 512, 24, 128, 1),
     (6, 512, 512, 24, 128, 3),

@@ -140,7 +140,7 @@ def test_stride_stages(DX, DY, nsig, tol):
     (1, 512, 512, 8, 64, 0),         # square, few images: X axis first
     (2, 512, 512, 64, 64, 0),        # square, K * bs = 128: whole rows first
     (1, 1024, 1024, 8, 64, 0),
-    (1, 128, 128, 16, 64, 3),        # whole rows first on every pair of lengths (row blocks of 32, 32, 32 and 16 rows)
+    (1, 128, 128, 16, 64, 3),        # whole rows first on every pair of lengths (row blocks of 32 rows, one to eight batches)
     (2, 256, 128, 8, 64, 3),
     (3, 128, 256, 24, 128, 3),
     (1, 256, 256, 72, 64, 3),

@@ -17,8 +17,8 @@ namespace tfno {
 
 template <int LOGDY> struct GeoRows {
     using G = Geo1D<LOGDY>;
-    static constexpr int BATCHES = LOGDY == 7 ? 1 : LOGDY == 8 ? 2 : 4;   // rows are transformed GROUPS at a time
-    static constexpr int ROWS = BATCHES * G::GROUPS;                  // rows of the image per block: 32, 32, 32, 16
+    static constexpr int BATCHES = LOGDY == 7 ? 1 : LOGDY == 8 ? 2 : LOGDY == 9 ? 4 : 8;   // rows are transformed GROUPS at a time
+    static constexpr int ROWS = BATCHES * G::GROUPS;                  // rows of the image per block: 32 at every length
     static constexpr int PT = ROWS + 1;                               // pitch (complex) of the tile [64][ROWS]
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(G::GROUPS * G::EXCH + 64 * PT);
 };
