@@ -107,3 +107,21 @@ def test_cgemm_beyond_65536_rows_per_channel(tol):
     picks = torch.tensor(sorted({0, 255, 256, 65535 * 256 - 1, 65535 * 256, M // 2 + 3, M - 257, M - 1}), device="cuda")
     ref = oracle.cgemm(A.index_select(1, picks).cpu().numpy(), W.cpu().numpy(), 1 - 1j)
     _check(C.index_select(1, picks).cpu().numpy(), ref, tol, "cgemm M=2^24")
+
+
+def test_row_kernels_beyond_65536_blocks(tol):
+    """2D layer with whole rows first on 66 x 8 input and 66 x 64 output images of 512 x 512: the backward row kernel runs
+    67,584 blocks (one per 32 rows), the forward row kernel walks 8,448 row blocks with its persistent grid; batch
+    elements on both sides of block 65,536 and the last one against the oracle"""
+    bs, D, K, N = 66, 512, 8, 64
+    print("large grid rows first", bs, D, K, N, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(91)
+    x = _uniform(gen, (K, bs, D, D))
+    W = _uniform(gen, (N, K))
+    y = tf.layer_2d(x, W, alpha=1 - 1j, algo=3)
+    torch.cuda.synchronize()
+    assert N * bs * (D // 32) > 65536
+    # output image n * bs + b is written by blocks 16 (n * bs + b) ... + 15: block 65,536 lies in image 4096 = (n 62, b 4)
+    for b in (0, 3, 4, 65):
+        ref = oracle.layer_2d(x[:, b:b + 1].cpu().numpy(), W.cpu().numpy(), 1 - 1j)
+        _check(y[:, b:b + 1].cpu().numpy(), ref, tol, "rows first bs=66 b=%d" % b)
