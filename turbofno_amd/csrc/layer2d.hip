@@ -314,25 +314,31 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
             for (int g = 0; g < NG; ++g)
                 bv[g] = (active && 4 * g < kn) ? (blk + (long)(kc + 4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
         }
-        __syncthreads();                              // the previous chunk's tile is no longer read
-        // W'' tile: lanes run along k, the contiguous direction of W[k + n*K]
-        constexpr int WPT = KCH * 64 / GEMM_THREADS;
-        float2 wv[WPT];
+        if constexpr (MULTI) __syncthreads();         // the previous chunk's tile is no longer read
+        // W'' tile: lanes run along k, the contiguous direction of W[k + n*K]. With a single chunk only the first
+        // BUILDERS threads build it: the waves of a block start one after the other over several microseconds, and the
+        // block can only go on when the last of them has passed the barrier below - which should then find nothing left
+        // to do there (its own part of the tile would add a round trip to L2 after its late start)
+        constexpr int BUILDERS = MULTI ? GEMM_THREADS : GEMM_THREADS / 2;
+        constexpr int WPT = KCH * 64 / BUILDERS;
+        if (MULTI || tid < BUILDERS) {
+            float2 wv[WPT];
 #pragma unroll
-        for (int u = 0; u < WPT; ++u) {
-            const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % KCH, n = idx / KCH;
-            wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
-        }
+            for (int u = 0; u < WPT; ++u) {
+                const int idx = tid + u * BUILDERS;
+                const int k = idx % KCH, n = idx / KCH;
+                wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+            }
 #pragma unroll
-        for (int u = 0; u < WPT; ++u) {
-            const int idx = tid + u * GEMM_THREADS;
-            const int k = idx % KCH, n = idx / KCH;
-            const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
-            float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
-            dstw[0] = c;
-            dstw[kW3Plane] = d - c;
-            dstw[2 * kW3Plane] = c + d;
+            for (int u = 0; u < WPT; ++u) {
+                const int idx = tid + u * BUILDERS;
+                const int k = idx % KCH, n = idx / KCH;
+                const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+                float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
+                dstw[0] = c;
+                dstw[kW3Plane] = d - c;
+                dstw[2 * kW3Plane] = c + d;
+            }
         }
         if constexpr (MULTI) {
 #pragma unroll
