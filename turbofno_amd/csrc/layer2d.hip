@@ -180,7 +180,18 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
 // Backward image kernel, mirror of the forward one: persistent blocks, 16 waves per CU, twiddles in LDS.
 // The 32 KiB spectrum of the next image is fetched (a few registers per lane) while the current image's rows
 // are being transformed and stored, so a CU never waits for its input between images.
-template <int LOGX, int LOGY>
+//
+// SHARE: the XCDs of this GPU do not store at the same rate. Workgroup b of a grid runs on XCD b mod 8, and the blocks on
+// the odd XCDs need about a fifth longer per image than those on the even ones (21.3 against 17.5 us at 256 x 256, in
+// every launch on every box measured; a store-only probe gives the same picture), so with the same number of images per
+// block the even half of the chip idles for the last sixth of the kernel. Here blocks 2p and 2p + 1 share the images
+// p, p + P, p + 2P, ... (P pairs) unevenly: of the J * ITY row passes of the pair's J images the even block takes a share
+// of kEvenShareNum / kEvenShareDen, in whole images plus the first row passes of one image that the two blocks split
+// (each takes it last; both run its column pass). 1024 images of 256 x 256: the even block transforms 4 1/4 images, the odd one 3 3/4: 101.6 -> 96.5 us.
+// Which row goes to which block does not change any value: the output is bit-identical to the equal split.
+constexpr int kEvenShareNum = 17, kEvenShareDen = 32;      // measured: 17/32 and 18/32 level (-5.3 us per layer), 19/32 -3 us
+
+template <int LOGX, int LOGY, bool SHARE>
 __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
                                                           int nimg)
 {
@@ -206,15 +217,42 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     const unsigned lane_off = (unsigned)(row0 * DY + ty);
     const bool col_thread = tid < G::COLT;
 
-    long img = blockIdx.x;
+    // The block transforms `count` images, image_at(k) for k < count; of its last one, if `split`, only the row passes
+    // [pass0, pass1). Without SHARE: every block the images blockIdx.x, + gridDim.x, ... in full.
+    long first = blockIdx.x, step = gridDim.x, last = 0;
+    int count = (int)((nimg - first + step - 1) / step), pass0 = 0, pass1 = ITY;
+    bool split = false;
+    if constexpr (SHARE) {
+        const int pairs = gridDim.x / 2, pr = blockIdx.x >> 1, odd = blockIdx.x & 1;     // the host launches an even grid
+        const int J = (nimg - pr + pairs - 1) / pairs;                                    // images of this pair
+        const int even_passes = (J * ITY * kEvenShareNum + kEvenShareDen / 2) / kEvenShareDen;
+        const int whole = even_passes / ITY, rest = even_passes % ITY;                    // of the even block
+        step = pairs;
+        split = rest != 0;
+        last = pr + (long)pairs * whole;                    // the image the pair splits: the last one of either block
+        if (!odd) {
+            first = pr;                                     // images 0 .. whole - 1 of the pair, then the first `rest` passes
+            count = whole + (split ? 1 : 0);
+            pass1 = rest;
+        } else {
+            first = pr + (long)pairs * (whole + (split ? 1 : 0));   // the pair's remaining whole images, then the other passes
+            count = J - whole;
+            pass0 = rest;
+        }
+    }
+    auto image_at = [&](int k) -> long { return (SHARE && split && k == count - 1) ? last : first + step * k; };
+
     cpx c[MMX];
-    if (img < nimg && col_thread) {
-        const float2* src = spec + img * 4096;
+    if (count > 0 && col_thread) {
+        const float2* src = spec + image_at(0) * 4096;
 #pragma unroll
         for (int mm = 0; mm < MMX; ++mm) c[mm] = src[tid + G::COLT * mm];
     }
-    for (; img < nimg; img += gridDim.x) {
-        const long pre = img + gridDim.x < nimg ? img + gridDim.x : img;
+    for (int k = 0; k < count; ++k) {
+        const long img = image_at(k);
+        const long pre = k + 1 < count ? image_at(k + 1) : img;
+        const bool partial = SHARE && split && k == count - 1;
+        const int it0 = partial ? pass0 : 0, it1 = partial ? pass1 : ITY;
         // pass 1: columns (p -> x) of column q = gx
         cpx u[16];
         if (col_thread) group_backward_lds<LOGX>(c, twrow_x, exch_x, tx, u);
@@ -241,6 +279,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
         // dirty lines from lingering in the Infinity Cache and being written back under the next kernel's reads
 #pragma unroll
         for (int it = 0; it < ITY; ++it) {
+            if (SHARE && (it < it0 || it >= it1)) continue;       // uniform: row passes of the split image left to the partner
             cpx yv[16];
             if constexpr (G::PAIRED) rows128_backward(cc[it], twrow_y, exch_y, ty, yv);
             else group_backward_lds<8>(cc[it], twrow_y, exch_y, ty, yv);
@@ -388,15 +427,22 @@ template <int LOGX, int LOGY>
 static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, int nimg, hipStream_t stream)
 {
     using G = Geo2D<LOGX, LOGY>;
-    static std::atomic<unsigned long long> served[2];
-    const void* fn = inverse ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY>)
-                             : reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>);
-    if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse]); e != hipSuccess) return e;
     // persistent blocks: at most as many as fit at once (LDS allows one or two 1024-thread blocks per CU,
     // the thread count exactly one)
     const int blocks = nimg < cu_count() ? nimg : cu_count();
-    if (inverse)
-        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
+    // uneven shares between the blocks of a pair: a full grid (one block per CU, so that block parity is XCD parity), at
+    // least two images per block (128 x 128 images are a single row pass each and are shared in whole images only)
+    const bool share = inverse && blocks == cu_count() && blocks % 2 == 0 && nimg >= 2 * blocks;
+    static std::atomic<unsigned long long> served[3];
+    const void* fn = !inverse ? reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>)
+                     : share ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, true>)
+                             : reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, false>);
+    if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse ? (share ? 2 : 1) : 0]); e != hipSuccess) return e;
+    if (share)
+        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, true>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
+                           out, nimg);
+    else if (inverse)
+        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, false>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
                            out, nimg);
     else
         hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
