@@ -35,6 +35,10 @@ __device__ __forceinline__ void decode_block_1d(long S, int ntiles, long& s, int
 }
 #endif
 
+// Share of the work of a pair of persistent blocks (2p on an even XCD, 2p + 1 on an odd one) that the even block takes in
+// the store-bound backward kernels: the odd XCDs of this GPU sustain about a fifth less store traffic than the even ones.
+constexpr int kEvenShareNum = 17, kEvenShareDen = 32;
+
 // compute units of the current device (cached per device)
 int cu_count();
 

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
 // of kEvenShareNum / kEvenShareDen, in whole images plus the first row passes of one image that the two blocks split
 // (each takes it last; both run its column pass). 1024 images of 256 x 256: the even block transforms 4 1/4 images, the odd one 3 3/4: 101.6 -> 96.5 us.
 // Which row goes to which block does not change any value: the output is bit-identical to the equal split.
-constexpr int kEvenShareNum = 17, kEvenShareDen = 32;      // measured: 17/32 and 18/32 level (-5.3 us per layer), 19/32 -3 us
+// (kEvenShareNum / kEvenShareDen in kernels.h; measured here: 17/32 and 18/32 level, -5.3 us per layer, 19/32 -3 us)
 
 template <int LOGX, int LOGY, bool SHARE>
 __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restrict__ spec, float2* __restrict__ y,

@@ -222,9 +222,22 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
         }
     };
     cpx c[NIN];
-    long panel = blockIdx.x;
-    if (panel < npanels) fetch(c, panel);
-    for (; panel < npanels; panel += gridDim.x) {
+    // The odd XCDs of this GPU store about a fifth slower than the even ones, and workgroup b runs on XCD b mod 8: the
+    // blocks 2p and 2p + 1 share the panels p, p + pairs, p + 2 pairs, ... of their pair 17 : 15 instead of evenly (the
+    // even block takes the first ones), so that both end together. An odd grid keeps the even split.
+    long panel = blockIdx.x, step = gridDim.x, last = npanels;
+    if ((gridDim.x & 1) == 0) {
+        const long pairs = gridDim.x >> 1, pr = blockIdx.x >> 1;
+        const long J = (npanels - pr + pairs - 1) / pairs;          // panels of this pair (pr < npanels: the grid is no larger)
+        const long even = (J * kEvenShareNum + kEvenShareDen / 2) / kEvenShareDen;
+        step = pairs;
+        panel = (blockIdx.x & 1) ? pr + pairs * even : pr;
+        last = (blockIdx.x & 1) ? npanels : pr + pairs * even;
+        if (last > npanels) last = npanels;
+    }
+    const long npanels_mine = last;
+    if (panel < npanels_mine) fetch(c, panel);
+    for (; panel < npanels_mine; panel += step) {
         const long col = panel * COLS + yl;
         const long sig = col / DY;
         const int y = (int)(col % DY);
@@ -250,7 +263,7 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
                 lds[(tt * 17 + t + 8) * COLS + yl] = h1[tt];
             }
         }
-        if (panel + gridDim.x < npanels) fetch(c, panel + gridDim.x);      // look-ahead: travels under the rest of this panel
+        if (panel + step < npanels_mine) fetch(c, panel + step);           // look-ahead: travels under the rest of this panel
         __syncthreads();
         cpx e[16], yv[16];
         if constexpr (L >= 32) {
