@@ -50,6 +50,35 @@ def test_layer_1d_beyond_65536_blocks(S, DY, K, N, algo, tol, algo_1d):
     _check(y.index_select(1, idx).cpu().numpy(), ref, tol, "layer_1d S=%d" % S)
 
 
+@pytest.mark.parametrize("S,DY,K,N,algo", [
+    (2048, 256, 8, 128, 0),          # 4 MiB between the rows of a signal set, two output tiles per set
+    (4096, 256, 16, 64, 3),          # 8 MiB, 256-thread matrix-core kernel
+    (4096, 128, 16, 64, 5),          # 4 MiB, one wavefront per item
+    (1024, 512, 8, 128, 0),          # 4 MiB at length 512
+    (512, 1024, 8, 64, 1),           # 4 MiB at length 1024, SIMT kernel
+    (2048, 256, 32, 256, 8),         # wide tiles, two per signal set
+    (8192, 256, 8, 64, 0),           # 16 MiB: the largest stride that takes this block order
+    (16384, 256, 8, 64, 0),          # 32 MiB: back to the interleaved order
+])
+def test_layer_1d_channel_strides_that_are_multiples_of_4MiB(S, DY, K, N, algo, tol, algo_1d):
+    """batch sizes for which XCD j walks the j-th eighth of the signal sets instead of every eighth set: every row of y
+    is written (y starts as NaN), and the sets at the seams of the eighths agree with the oracle"""
+    print("power-of-two stride layer_1d", S, DY, K, N, algo, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(S + DY + K)
+    x = _uniform(gen, (K, S, DY))
+    W = _uniform(gen, (N, K)) / np.sqrt(K)
+    y = torch.full((N, S, DY), float("nan"), dtype=torch.complex64, device="cuda")
+    algo_1d(algo)
+    tf.layer_1d(x, W, y=y, alpha=0.5 + 1j)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(torch.view_as_real(y)).any()), "rows of y left unwritten"
+    e = S // 8
+    picks = sorted({0, 1, 7, 8, e - 1, e, e + 1, 3 * e - 1, 3 * e, S // 2, 7 * e - 1, 7 * e, S - 2, S - 1})
+    idx = torch.tensor(picks, device="cuda")
+    ref = oracle.layer_1d(x.index_select(1, idx).cpu().numpy(), W.cpu().numpy(), 0.5 + 1j)
+    _check(y.index_select(1, idx).cpu().numpy(), ref, tol, "layer_1d S=%d DY=%d" % (S, DY))
+
+
 @pytest.mark.parametrize("DX,DY,nsig", [(128, 256, 8300), (256, 128, 16500)])
 def test_stride_kernels_beyond_65536_blocks(DX, DY, nsig, tol):
     """X-axis kernels: nsig * DY / 16 (forward) and nsig * DY / 32 (backward) blocks, both above 65,536"""
