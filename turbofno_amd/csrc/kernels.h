@@ -27,14 +27,20 @@ constexpr int kWGroup = 1032;
 // HBM peak, S = 4096 0.61, S = 3584 0.70). For these strides XCD j walks the j-th eighth of the signal sets instead
 // (tiles of a signal set on consecutive blocks of that XCD): S = 2048 0.65, S = 4096 0.71; up to -26 % at DY = 512.
 // Up to a stride of 16 MiB; beyond it the grids are large enough to hide the effect and the contiguous walk costs 2-5 %.
+// Only for launches that stream x from and y to HBM (`streamed`): as the middle stage of a 2D pipeline, with its input
+// and output in the caches, the same kernels are a quarter SLOWER in that order (16 images of 512 x 512: layer 750 ->
+// 778 us), and keep the interleaved one.
+// Workgroup b of a one-dimensional grid runs on XCD b mod 8: renumbered like this, XCD j takes the j-th eighth of n
+// work items, in order, instead of every eighth item.
+__device__ __forceinline__ long xcd_contiguous(long b, long n) { return (n & 7) == 0 ? (b & 7) * (n >> 3) + (b >> 3) : b; }
 __host__ __device__ __forceinline__ bool xcd_walks_an_eighth_1d(long S, int DY)
 {
     const long stride = S * DY * 8;
     return stride % (4L << 20) == 0 && stride <= (16L << 20);      // S is then a multiple of 8
 }
-__device__ __forceinline__ void decode_block_1d(long S, int ntiles, int DY, long& s, int& tile)
+__device__ __forceinline__ void decode_block_1d(long S, int ntiles, int DY, bool streamed, long& s, int& tile)
 {
-    if (xcd_walks_an_eighth_1d(S, DY)) {
+    if (streamed && xcd_walks_an_eighth_1d(S, DY)) {
         const long id = blockIdx.x, q = id >> 3;
         s = (id & 7) * (S / 8) + q / ntiles;
         tile = (int)(q % ntiles);

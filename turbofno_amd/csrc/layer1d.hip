@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void fused_fft_cgemm_ifft_kernel(int S, int N,
     const int g = tid / L, t = tid % L;
     long s;
     int ntile;
-    decode_block_1d(S, N / 64, 1 << LOGDY, s, ntile);
+    decode_block_1d(S, N / 64, 1 << LOGDY, !KEEP, s, ntile);
     const int n0 = ntile * 64;
     const long M = 64L * S;
     // signals of 128 samples are transformed in pairs by 16-lane groups (128-byte accesses): lane t16 of pair g/2 holds
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     const int mt = wave & 3, nt0 = (wave >> 2) * NTW;          // m tile, first of the wave's NTW n' tiles
     long s;
     int ntile;
-    decode_block_1d(S, N / NT, 1 << LOGDY, s, ntile);
+    decode_block_1d(S, N / NT, 1 << LOGDY, !KEEP, s, ntile);
     const int n0 = ntile * NT;
     // DY = 128: signals are transformed in pairs by 16-lane groups (see the SIMT kernel); COMPACT never applies there
     constexpr bool PAIR = LOGDY == 7;
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     __syncthreads();
     long s;
     int ntile;
-    decode_block_1d(S, N / 64, 1 << LOGDY, s, ntile);
+    decode_block_1d(S, N / 64, 1 << LOGDY, !KEEP, s, ntile);
     const int n0 = ntile * 64;
     const bool upper = t >> 3, odd = t & 1;
 
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_split_kernel(int S, i
     float2* exch = lds + (4 * w + g) * EXCH;                      // the partials overlay these after the K loop
     long s;
     int ntile;
-    decode_block_1d(S, N / SPLIT_NT, 256, s, ntile);
+    decode_block_1d(S, N / SPLIT_NT, 256, true, s, ntile);
     const int n0 = ntile * SPLIT_NT;
     const bool odd = t & 1;
     cpx tw[16];

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide_kernel(int S,
     const int mt = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;     // matrix role: m tile = wave
     long s;
     int ntile;
-    decode_block_1d(S, N / NT, 256, s, ntile);
+    decode_block_1d(S, N / NT, 256, !KEEP, s, ntile);
     const int n0 = ntile * NT;
     float2* exch = lds + g * G::EXCH;
 
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256, 2) void fused_fft_mfma_ifft_wide128_kernel(int
     const int mt = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;     // matrix role: m tile = wave
     long s;
     int ntile;
-    decode_block_1d(S, N / NT, 128, s, ntile);
+    decode_block_1d(S, N / NT, 128, !KEEP, s, ntile);
     const int n0 = ntile * NT;
     float2* exch = lds + grp * G::EXCH;
 

@@ -330,9 +330,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.y * 64;
     const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
-    const float2* blk = A + (long)blockIdx.x * GEMM_MBLOCK;
-    const bool active = (long)blockIdx.x * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
-    float2* cblk = C + (long)blockIdx.x * GEMM_MBLOCK;
+    // XCD j takes the j-th eighth of the column blocks: with every eighth block (2 KiB of each of the K + N rows, which
+    // lie Mtot * 8 bytes apart) an XCD keeps to one part of the memory system; 4-10 % faster once the operands exceed the
+    // Infinity Cache (bs = 128), no change below
+    const unsigned mb = (unsigned)xcd_contiguous(blockIdx.x, gridDim.x);
+    const float2* blk = A + (long)mb * GEMM_MBLOCK;
+    const bool active = (long)mb * GEMM_MBLOCK + wave * 16 < Mtot;   // Mtot is a multiple of 16, not of 256
+    float2* cblk = C + (long)mb * GEMM_MBLOCK;
     const bool has_beta = beta.x != 0.f || beta.y != 0.f;
 
     floatx4 p1[4], p2[4], p3[4];
