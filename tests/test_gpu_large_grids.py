@@ -57,6 +57,8 @@ def test_layer_1d_beyond_65536_blocks(S, DY, K, N, algo, tol, algo_1d):
     (1024, 512, 8, 128, 0),          # 4 MiB at length 512
     (512, 1024, 8, 64, 1),           # 4 MiB at length 1024, SIMT kernel
     (2048, 256, 32, 256, 8),         # wide tiles, two per signal set
+    (2048, 256, 64, 64, 6),          # eight waves split the channels of an item, two 32-channel tiles per signal set
+    (2048, 256, 64, 128, 2),         # 512-thread matrix-core kernel
     (8192, 256, 8, 64, 0),           # 16 MiB: the largest stride that takes this block order
     (16384, 256, 8, 64, 0),          # 32 MiB: back to the interleaved order
 ])
