@@ -81,6 +81,33 @@ def test_layer_1d_channel_strides_that_are_multiples_of_4MiB(S, DY, K, N, algo, 
     _check(y.index_select(1, idx).cpu().numpy(), ref, tol, "layer_1d S=%d DY=%d" % (S, DY))
 
 
+@pytest.mark.parametrize("M,K,N,beta", [
+    (131072, 64, 64, 0.0),           # 512 column blocks: two per CU, the walk in eighths
+    (131072 + 192, 24, 128, 0.0),    # a partly filled last column block, two n tiles, 513 column blocks (plain walk)
+    (262144, 40, 64, 0.25 - 0.5j),   # four per CU, C read and written (beta)
+])
+def test_cgemm_with_several_column_blocks_per_cu(M, K, N, beta, tol):
+    """the mode GEMM as persistent blocks that walk the column blocks: every column written (C starts as NaN when beta
+    is zero), columns at the start, at the seams of the eighths and at the end against the oracle"""
+    print("persistent cgemm", M, K, N, beta, flush=True)
+    gen = torch.Generator(device="cuda").manual_seed(M + K)
+    A = _uniform(gen, (K, M))
+    W = _uniform(gen, (N, K)) / np.sqrt(K)
+    C0 = _uniform(gen, (N, M)) if beta != 0.0 else torch.full((N, M), float("nan"), dtype=torch.complex64, device="cuda")
+    C = C0.clone()
+    tf.cgemm(M, N, K, A, W, C, 0.5 + 1j, beta)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(torch.view_as_real(C)).any()), "columns of C left unwritten"
+    seam = (M // 256 // 8) * 256
+    picks = sorted(set(list(range(0, 40)) + list(range(seam - 20, seam + 20)) + list(range(5 * seam - 20, 5 * seam + 20))
+                       + list(range(M // 2, M // 2 + 16)) + list(range(M - 300, M))))
+    idx = torch.tensor(picks, device="cuda")
+    ref = oracle.cgemm(A.index_select(1, idx).cpu().numpy(), W.cpu().numpy(), 0.5 + 1j)
+    if beta != 0.0:
+        ref = ref + beta * C0.index_select(1, idx).cpu().numpy().astype(np.complex128)
+    _check(C.index_select(1, idx).cpu().numpy(), ref, tol, "cgemm M=%d K=%d N=%d" % (M, K, N))
+
+
 @pytest.mark.parametrize("DX,DY,nsig", [(128, 256, 8300), (256, 128, 16500)])
 def test_stride_kernels_beyond_65536_blocks(DX, DY, nsig, tol):
     """X-axis kernels: nsig * DY / 16 (forward) and nsig * DY / 32 (backward) blocks, both above 65,536"""

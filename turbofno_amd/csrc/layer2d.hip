@@ -415,6 +415,88 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
     }
 }
 
+// K <= 64 and several column blocks per CU: persistent. A block builds the W'' tile once and walks column blocks (XCD j the
+// j-th eighth of them, in order). There is no barrier inside the walk, so the waves of a CU drift apart, and the loads of
+// one, the matrix work of another and the stores of a third overlap; the strip of the next column block is requested
+// before the matrix work on the current one starts. (With one column block per CU this is the kernel above.)
+template <int NG>
+__global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(const float2* __restrict__ A,
+                                                                                const float2* __restrict__ W,
+                                                                                float2* __restrict__ C, long Mtot, int N, int K,
+                                                                                float2 alpha, float2 beta, long nblocks)
+{
+    extern __shared__ float sW[];                     // 3 * kW3Plane floats
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.y * 64;
+    const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
+    const bool has_beta = beta.x != 0.f || beta.y != 0.f;
+    const bool eighths = (gridDim.x & 7) == 0 && (nblocks & 7) == 0;
+    auto block_of = [&](long v) { return eighths ? (v & 7) * (nblocks >> 3) + (v >> 3) : v; };
+    auto fetch = [&](float2 (&dst)[NG], long mb) {
+        const bool active = mb * GEMM_MBLOCK + wave * 16 < Mtot;      // Mtot is a multiple of 16, not of 256
+        const float2* blk = A + mb * GEMM_MBLOCK;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) dst[g] = (active && 4 * g < K) ? (blk + (long)(4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+    };
+    long v = blockIdx.x;                              // the grid is no larger than the number of column blocks
+    float2 bv[NG];
+    fetch(bv, block_of(v));
+    {
+        constexpr int WPT = GEMM_KC * 64 / GEMM_THREADS;
+        float2 wv[WPT];
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+            wv[u] = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < WPT; ++u) {
+            const int idx = tid + u * GEMM_THREADS;
+            const int k = idx % GEMM_KC, n = idx / GEMM_KC;
+            const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
+            float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
+            dstw[0] = c;
+            dstw[kW3Plane] = d - c;
+            dstw[2 * kW3Plane] = c + d;
+        }
+    }
+    __syncthreads();
+    for (; v < nblocks; v += gridDim.x) {
+        asm volatile("" ::: "memory");                // keeps the operand fetches from the W'' tile inside the loop (192 registers otherwise)
+        const long mb = block_of(v);
+        const bool more = v + gridDim.x < nblocks;
+        const long nb = more ? block_of(v + gridDim.x) : mb;
+        const bool next_active = more && nb * GEMM_MBLOCK + wave * 16 < Mtot;
+        const float2* nblk = A + nb * GEMM_MBLOCK;
+        const bool active = mb * GEMM_MBLOCK + wave * 16 < Mtot;
+        float2* cblk = C + mb * GEMM_MBLOCK;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            floatx4 p1 = floatx4{ 0.f, 0.f, 0.f, 0.f }, p2 = p1, p3 = p1;
+            const float* wrow = &sW[kq * kW3Row + t * 16 + col];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                const float* w = wrow + g * kW3Group;
+                p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0], bv[g].x + bv[g].y, p1, 0, 0, 0);
+                p2 = __builtin_amdgcn_mfma_f32_16x16x4f32(w[kW3Plane], bv[g].x, p2, 0, 0, 0);
+                p3 = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * kW3Plane], bv[g].y, p3, 0, 0, 0);
+                // the last n tile has used this group of the strip: its registers take the next column block's
+                if (t == 3 && more) bv[g] = (next_active && 4 * g < K) ? (nblk + (long)(4 * g) * Mtot)[lane_off] : make_float2(0.f, 0.f);
+            }
+            if (active) {
+#pragma unroll
+                for (int vv = 0; vv < 4; ++vv) {
+                    float2* p = cblk + (long)(n0 + 16 * t + 4 * kq + vv) * Mtot + (wave * 16 + col);
+                    float2 r = make_float2(p1[vv] - p3[vv], p1[vv] + p2[vv]);
+                    if (has_beta) r = cadd(r, cmul(*p, beta));      // C = alpha A W + beta C (variants A, B)
+                    *p = r;
+                }
+            }
+        }
+    }
+}
+
 int cu_count()
 {
     static std::atomic<int> cached[64];
@@ -491,6 +573,28 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
                            alpha, beta);
         return hipGetLastError();
     };
+    // several column blocks per CU, one chunk: persistent blocks, one per CU (and n tile)
+    auto launch_persistent = [&](auto ng_const) -> hipError_t {
+        constexpr int NG = decltype(ng_const)::value;
+        static std::atomic<unsigned long long> served;
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_persistent_kernel<NG>), lds_bytes, served);
+            e != hipSuccess)
+            return e;
+        const long nblocks = grid.x;
+        long g = cu_count();
+        if (g >= 8) g -= g % 8;                                  // whole groups of eight: every XCD the same share
+        hipLaunchKernelGGL((cgemm_modes3m_persistent_kernel<NG>), dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), lds_bytes,
+                           stream, A, W, C, Mtot, N, K, alpha, beta, nblocks);
+        return hipGetLastError();
+    };
+    // from two column blocks per CU (K = N = 64: M = 131,072 40 -> 37 us, 262,144 75 -> 64, 524,288 164 -> 133; below that
+    // the two kernels are level)
+    if (K <= GEMM_KC && (long)grid.x >= 2L * cu_count()) {
+        if (K <= 16) return launch_persistent(std::integral_constant<int, 4>{});
+        if (K <= 32) return launch_persistent(std::integral_constant<int, 8>{});
+        if (K <= 48) return launch_persistent(std::integral_constant<int, 12>{});
+        return launch_persistent(std::integral_constant<int, 16>{});
+    }
     if (K <= 16) return launch(std::integral_constant<int, 4>{}, std::false_type{});
     if (K <= 32) return launch(std::integral_constant<int, 8>{}, std::false_type{});
     if (K <= 48) return launch(std::integral_constant<int, 12>{}, std::false_type{});
