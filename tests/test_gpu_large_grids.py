@@ -84,7 +84,8 @@ def test_layer_1d_channel_strides_that_are_multiples_of_4MiB(S, DY, K, N, algo, 
 @pytest.mark.parametrize("M,K,N,beta", [
     (131072, 64, 64, 0.0),           # 512 column blocks: two per CU, the walk in eighths
     (131072 + 192, 24, 128, 0.0),    # a partly filled last column block, two n tiles, 513 column blocks (plain walk)
-    (262144, 40, 64, 0.25 - 0.5j),   # four per CU, C read and written (beta)
+    (262144, 40, 64, 0.0),           # four per CU
+    (262144, 40, 64, 0.25 - 0.5j),   # C read and written (beta): the kernel with one column block per block
 ])
 def test_cgemm_with_several_column_blocks_per_cu(M, K, N, beta, tol):
     """the mode GEMM as persistent blocks that walk the column blocks: every column written (C starts as NaN when beta

@@ -418,18 +418,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
 // K <= 64 and several column blocks per CU: persistent. A block builds the W'' tile once and walks column blocks (XCD j the
 // j-th eighth of them, in order). There is no barrier inside the walk, so the waves of a CU drift apart, and the loads of
 // one, the matrix work of another and the stores of a third overlap; the strip of the next column block is requested
-// before the matrix work on the current one starts. (With one column block per CU this is the kernel above.)
+// before the matrix work on the current one starts. C = alpha A W only (beta = 0).
 template <int NG>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(const float2* __restrict__ A,
                                                                                 const float2* __restrict__ W,
                                                                                 float2* __restrict__ C, long Mtot, int N, int K,
-                                                                                float2 alpha, float2 beta, long nblocks)
+                                                                                float2 alpha, long nblocks)
 {
     extern __shared__ float sW[];                     // 3 * kW3Plane floats
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.y * 64;
     const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
-    const bool has_beta = beta.x != 0.f || beta.y != 0.f;
     const bool eighths = (gridDim.x & 7) == 0 && (nblocks & 7) == 0;
     auto block_of = [&](long v) { return eighths ? (v & 7) * (nblocks >> 3) + (v >> 3) : v; };
     auto fetch = [&](float2 (&dst)[NG], long mb) {
@@ -488,9 +487,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(
 #pragma unroll
                 for (int vv = 0; vv < 4; ++vv) {
                     float2* p = cblk + (long)(n0 + 16 * t + 4 * kq + vv) * Mtot + (wave * 16 + col);
-                    float2 r = make_float2(p1[vv] - p3[vv], p1[vv] + p2[vv]);
-                    if (has_beta) r = cadd(r, cmul(*p, beta));      // C = alpha A W + beta C (variants A, B)
-                    *p = r;
+                    *p = make_float2(p1[vv] - p3[vv], p1[vv] + p2[vv]);
                 }
             }
         }
@@ -584,12 +581,14 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         long g = cu_count();
         if (g >= 8) g -= g % 8;                                  // whole groups of eight: every XCD the same share
         hipLaunchKernelGGL((cgemm_modes3m_persistent_kernel<NG>), dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), lds_bytes,
-                           stream, A, W, C, Mtot, N, K, alpha, beta, nblocks);
+                           stream, A, W, C, Mtot, N, K, alpha, nblocks);
         return hipGetLastError();
     };
     // from two column blocks per CU (K = N = 64: M = 131,072 40 -> 37 us, 262,144 75 -> 64, 524,288 164 -> 133; below that
     // the two kernels are level)
-    if (K <= GEMM_KC && (long)grid.x >= 2L * cu_count()) {
+    // Not with beta: reading C back inside the walk waits for the strip requested just before it (K = 32, M = 262,144:
+    // 79 against 74 us).
+    if (K <= GEMM_KC && (long)grid.x >= 2L * cu_count() && beta.x == 0.f && beta.y == 0.f) {
         if (K <= 16) return launch_persistent(std::integral_constant<int, 4>{});
         if (K <= 32) return launch_persistent(std::integral_constant<int, 8>{});
         if (K <= 48) return launch_persistent(std::integral_constant<int, 12>{});
