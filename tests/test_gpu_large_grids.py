@@ -85,6 +85,8 @@ def test_layer_1d_channel_strides_that_are_multiples_of_4MiB(S, DY, K, N, algo, 
     (131072, 64, 64, 0.0),           # 512 column blocks: two per CU, the walk in eighths
     (131072 + 192, 24, 128, 0.0),    # a partly filled last column block, two n tiles, 513 column blocks (plain walk)
     (262144, 40, 64, 0.0),           # four per CU
+    (65536, 64, 128, 0.0),           # two n tiles share the CUs: 128 blocks per n tile, two column blocks each
+    (65536 + 64, 48, 192, 0.0),      # three n tiles, a partly filled last column block
     (262144, 40, 64, 0.25 - 0.5j),   # C read and written (beta): the kernel with one column block per block
 ])
 def test_cgemm_with_several_column_blocks_per_cu(M, K, N, beta, tol):

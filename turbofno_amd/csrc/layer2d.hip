@@ -578,8 +578,13 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
             e != hipSuccess)
             return e;
         const long nblocks = grid.x;
+        // one block per CU and n tile; with several n tiles, 48 channels or more and up to two column blocks per CU the
+        // matrix pipes are the bound and one block per CU in all is faster (N = 128, K = 64: M = 65,536 41 -> 35 us,
+        // 131,072 71 -> 62; with fewer channels or more columns the kernel is bound by the loads in flight and loses 5-25 %)
         long g = cu_count();
+        if (grid.y > 1 && K >= 48 && nblocks <= 2L * cu_count()) g /= (long)grid.y;
         if (g >= 8) g -= g % 8;                                  // whole groups of eight: every XCD the same share
+        if (g < 1) g = 1;
         hipLaunchKernelGGL((cgemm_modes3m_persistent_kernel<NG>), dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), lds_bytes,
                            stream, A, W, C, Mtot, N, K, alpha, nblocks);
         return hipGetLastError();
@@ -588,7 +593,8 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
     // the two kernels are level)
     // Not with beta: reading C back inside the walk waits for the strip requested just before it (K = 32, M = 262,144:
     // 79 against 74 us).
-    if (K <= GEMM_KC && (long)grid.x >= 2L * cu_count() && beta.x == 0.f && beta.y == 0.f) {
+    if (K <= GEMM_KC && beta.x == 0.f && beta.y == 0.f &&
+        ((long)grid.x >= 2L * cu_count() || (K >= 48 && (long)grid.x * (long)grid.y >= 2L * cu_count()))) {
         if (K <= 16) return launch_persistent(std::integral_constant<int, 4>{});
         if (K <= 32) return launch_persistent(std::integral_constant<int, 8>{});
         if (K <= 48) return launch_persistent(std::integral_constant<int, 12>{});
