@@ -207,12 +207,9 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
 
     cpx tw[16];
     const float2* twrow = lds + G::REGION0 + G::REGION1 + t * kTwLdsPitch;
-    // compact: this thread's entry of the 16 x 16 twiddle table; requested before the first rows of x, stored after
-    // they have been requested
-    cpx tw_entry;
     if constexpr (G::COMPACT) {
-        static_assert(!G::COMPACT || THREADS == 256, "one table entry per thread");
-        tw_entry = kTwiddle1024[(((tid >> 4) * (tid & 15)) << (10 - LOGDY)) & 1023];
+        fill_lds_twiddles<LOGDY>(lds + G::REGION0 + G::REGION1, tid, THREADS);
+        __syncthreads();
     } else {
         load_lane_twiddles<LOGDY>(PAIR ? t16 : t, tw);
     }
@@ -237,12 +234,6 @@ __global__ __launch_bounds__(THREADS, (THREADS == 256 && LOGDY == 8) ? 3 : 1) vo
     cpx v0[16], v1[16];
     if (g < K) issue(v0, 0);
     if (G::DEPTH == 2 && KC + g < K) issue(v1, KC);
-    if constexpr (G::COMPACT) {
-        // The table entry arrives before the rows of x (loads return in order). The block meets on the LDS stores only:
-        // a full barrier would also wait for the rows, whose latency the first chunk's W loads and this store now cover.
-        lds[G::REGION0 + G::REGION1 + (tid >> 4) * kTwLdsPitch + (tid & 15)] = tw_entry;
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    }
 
     auto chunk = [&](cpx (&v)[16], int kc) {
         const int kn = (K - kc) < KC ? (K - kc) : KC;          // multiple of 8 (caller contract)
