@@ -87,6 +87,8 @@ def test_layer_1d_channel_strides_that_are_multiples_of_4MiB(S, DY, K, N, algo, 
     (262144, 40, 64, 0.0),           # four per CU
     (65536, 64, 128, 0.0),           # two n tiles share the CUs: 128 blocks per n tile, two column blocks each
     (65536 + 64, 48, 192, 0.0),      # three n tiles, a partly filled last column block
+    (262144, 104, 128, 0.0),         # more than 64 channels, eight column blocks per CU: the whole W tile in LDS, chunks of 32
+    (524288 + 128, 72, 64, 0.0),     # the same with one n tile and a partly filled last column block
     (262144, 40, 64, 0.25 - 0.5j),   # C read and written (beta): the kernel with one column block per block
 ])
 def test_cgemm_with_several_column_blocks_per_cu(M, K, N, beta, tol):

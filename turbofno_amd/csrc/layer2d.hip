@@ -494,6 +494,83 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(
     }
 }
 
+// 64 < K <= 128, beta = 0: persistent as well. The W'' tile of ALL channels (three planes of 32 channel groups, 123 KiB:
+// one block per CU) is built once; a column block is multiplied in chunks of 32 channels with the accumulators of the
+// four n tiles kept, the strip registers of a chunk take the next chunk (or the first chunk of the next column block) as
+// soon as the last n tile has used them, and nothing inside the walk waits at a barrier.
+constexpr int GEMM_KMAX = 128;
+constexpr int kW3WidePlane = (GEMM_KMAX / 4) * kW3Group;
+__global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_wide_kernel(const float2* __restrict__ A,
+                                                                                     const float2* __restrict__ W,
+                                                                                     float2* __restrict__ C, long Mtot, int N, int K,
+                                                                                     float2 alpha, long nblocks)
+{
+    extern __shared__ float sW[];                     // 3 * kW3WidePlane floats
+    constexpr int NG = 8;                             // channel groups per chunk
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.y * 64;
+    const unsigned lane_off = (unsigned)(kq * Mtot) + (unsigned)(wave * 16 + col);
+    const bool eighths = (gridDim.x & 7) == 0 && (nblocks & 7) == 0;
+    auto block_of = [&](long v) { return eighths ? (v & 7) * (nblocks >> 3) + (v >> 3) : v; };
+    const int nchunks = (K + 4 * NG - 1) / (4 * NG);
+    // strip of chunk c of column block mb: lane (kq, col) holds channels 32 c + 4 g + kq
+    auto strip_elem = [&](long mb, int c, int g) {
+        const int k = 4 * NG * c + 4 * g;
+        const bool ok = mb * GEMM_MBLOCK + wave * 16 < Mtot && k < K;         // Mtot is a multiple of 16, not of 256
+        return ok ? (A + mb * GEMM_MBLOCK + (long)k * Mtot)[lane_off] : make_float2(0.f, 0.f);
+    };
+    long v = blockIdx.x;                              // the grid is no larger than the number of column blocks
+    float2 bv[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) bv[g] = strip_elem(block_of(v), 0, g);
+    for (int idx = tid; idx < GEMM_KMAX * 64; idx += GEMM_THREADS) {
+        const int k = idx % GEMM_KMAX, n = idx / GEMM_KMAX;
+        const float2 w = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        const float c = w.x * alpha.x - w.y * alpha.y, d = w.x * alpha.y + w.y * alpha.x;
+        float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
+        dstw[0] = c;
+        dstw[kW3WidePlane] = d - c;
+        dstw[2 * kW3WidePlane] = c + d;
+    }
+    __syncthreads();
+    for (; v < nblocks; v += gridDim.x) {
+        asm volatile("" ::: "memory");                // keeps the operand fetches from the W'' tile inside the loop
+        const long mb = block_of(v);
+        const bool more = v + gridDim.x < nblocks;
+        const long nb = more ? block_of(v + gridDim.x) : mb;
+        floatx4 p1[4], p2[4], p3[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) p1[t] = p2[t] = p3[t] = floatx4{ 0.f, 0.f, 0.f, 0.f };
+        for (int c = 0; c < nchunks; ++c) {
+            const bool last = c + 1 == nchunks;
+            const bool refill = !last || more;
+            const long fb = last ? nb : mb;           // where the strip registers are refilled from
+            const int fc = last ? 0 : c + 1;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float* wrow = &sW[(c * NG) * kW3Group + kq * kW3Row + t * 16 + col];
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    const float* w = wrow + g * kW3Group;
+                    p1[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0], bv[g].x + bv[g].y, p1[t], 0, 0, 0);
+                    p2[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[kW3WidePlane], bv[g].x, p2[t], 0, 0, 0);
+                    p3[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * kW3WidePlane], bv[g].y, p3[t], 0, 0, 0);
+                    if (t == 3 && refill) bv[g] = strip_elem(fb, fc, g);
+                }
+            }
+        }
+        if (mb * GEMM_MBLOCK + wave * 16 < Mtot) {
+            float2* cblk = C + mb * GEMM_MBLOCK;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int vv = 0; vv < 4; ++vv)
+                    cblk[(long)(n0 + 16 * t + 4 * kq + vv) * Mtot + (wave * 16 + col)] =
+                        make_float2(p1[t][vv] - p3[t][vv], p1[t][vv] + p2[t][vv]);
+        }
+    }
+}
+
 int cu_count()
 {
     static std::atomic<int> cached[64];
@@ -599,6 +676,22 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         if (K <= 32) return launch_persistent(std::integral_constant<int, 8>{});
         if (K <= 48) return launch_persistent(std::integral_constant<int, 12>{});
         return launch_persistent(std::integral_constant<int, 16>{});
+    }
+    // from eight column blocks per CU (all n tiles together): 3-9 % ahead of the chunked kernel below (K = N = 128,
+    // M = 262,144: 274 -> 255 us); level at four, and up to 8 % behind on small problems (the larger tile to build)
+    if (K > GEMM_KC && K <= GEMM_KMAX && beta.x == 0.f && beta.y == 0.f && (long)grid.x * (long)grid.y >= 8L * cu_count()) {
+        constexpr size_t wide_lds = sizeof(float) * 3 * kW3WidePlane;            // 123,264 B: one block per CU
+        static std::atomic<unsigned long long> served;
+        if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(cgemm_modes3m_persistent_wide_kernel), wide_lds, served);
+            e != hipSuccess)
+            return e;
+        long g = cu_count() / (long)grid.y;
+        if (g >= 8) g -= g % 8;
+        if (g < 1) g = 1;
+        if (g > (long)grid.x) g = grid.x;
+        hipLaunchKernelGGL(cgemm_modes3m_persistent_wide_kernel, dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), wide_lds, stream, A,
+                           W, C, Mtot, N, K, alpha, (long)grid.x);
+        return hipGetLastError();
     }
     if (K <= 16) return launch(std::integral_constant<int, 4>{}, std::false_type{});
     if (K <= 32) return launch(std::integral_constant<int, 8>{}, std::false_type{});
