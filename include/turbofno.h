@@ -84,7 +84,8 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:133-172). The reference keeps its
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
- * algo: TURBOFNO_2D_AUTO picks WHOLE_IMAGE once K*bs images fill the CUs, THREE_KERNEL below; the workspace query
+ * algo: TURBOFNO_2D_AUTO picks by size (lengths up to 256: WHOLE_IMAGE from a batch of 8, and from a batch of 4 when
+ * there are enough images; THREE_KERNEL below; longer axes: ROWS_FIRST or THREE_KERNEL); the workspace query
  * with the same arguments makes the same choice. ROWS_FIRST is the three-stage structure with the axes exchanged
  * (the contiguous axis is transformed first and last, so that x and y move as whole rows): same result, the 2D
  * transform being separable; its intermediates are [images][64][DX].

@@ -50,15 +50,14 @@ int check_gemm_dims(long M, int N, int K)
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-// AUTO: the whole-image path runs one persistent block per image, so it needs enough input images (K*bs) to occupy
-// the CUs; below that the three-kernel path spreads an image over many blocks and is faster although it moves 1.5x
-// the bytes. Measured crossover on MI355X (256 CUs): one input image per CU, and for images smaller than 256 x 256
-// also a batch of at least 8 (with fewer, the three launches of the other path finish sooner). N does not enter: with
-// half an input image per CU and the output images filling the grid twice the two paths are within a few percent of each
-// other (bs = 8, K = 16, 256 x 256: 85 vs 91 us at N = 64, 144 vs 140 us at N = 128).
+// AUTO: the whole-image path runs one persistent block per image and moves 2/3 of the bytes of the three-kernel path,
+// which in turn spreads an image over many blocks and gets three short launches through sooner when there are few
+// images. Measured on MI355X (256 CUs; 160 shapes, both paths back to back): from a batch of 8 the whole-image path is
+// ahead (by up to 2x at bs = 16) but for two groups of shapes (below); with a batch of 4 to 7 it is ahead for 256 x 256
+// images once (K + N) * bs reaches 768 images in and out, and for 128 x 256 images with N >= 128; below a batch of 4 the
+// three-kernel path is 12-100 % ahead everywhere.
 int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
-    (void)N;
     if (algo != TURBOFNO_2D_AUTO) return algo;
     if (DX > 256 || DY > 256) {
         // an image no longer fits one block's LDS: three stages. The axis that is transformed first is the one whose
@@ -67,10 +66,18 @@ int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
         if (DY != DX) return DY > DX ? TURBOFNO_2D_ROWS_FIRST : TURBOFNO_2D_THREE_KERNEL;
         return (DY >= 1024 || (long)K * bs >= 128) ? TURBOFNO_2D_ROWS_FIRST : TURBOFNO_2D_THREE_KERNEL;
     }
-    const long in_images = (long)K * bs;
+    if (bs >= 16) return TURBOFNO_2D_WHOLE_IMAGE;
+    if (bs < 4) return TURBOFNO_2D_THREE_KERNEL;
     const bool big = DX == 256 && DY == 256;
-    const bool enough = in_images >= 256;
-    return (enough && (big || bs >= 8)) ? TURBOFNO_2D_WHOLE_IMAGE : TURBOFNO_2D_THREE_KERNEL;
+    if (bs >= 8) {
+        // two exceptions measured 7-13 % behind: few images of 256 x 256, and 256 x 128 images with 64 output channels
+        if (big && ((long)K + N) * bs < 768) return TURBOFNO_2D_THREE_KERNEL;
+        if (DX == 256 && DY == 128 && N == 64 && K < 128) return TURBOFNO_2D_THREE_KERNEL;
+        return TURBOFNO_2D_WHOLE_IMAGE;
+    }
+    if (big && ((long)K + N) * bs >= 768) return TURBOFNO_2D_WHOLE_IMAGE;
+    if (DX == 128 && DY == 256 && N >= 128) return TURBOFNO_2D_WHOLE_IMAGE;
+    return TURBOFNO_2D_THREE_KERNEL;
 }
 
 }  // namespace
