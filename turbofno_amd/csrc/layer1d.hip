@@ -788,6 +788,24 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
         if (blocks > cu_count() && blocks <= 64L * cu_count() && 4 * blocks >= 3 * rounds * slots)
             return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
     }
+    // DY = 128, about one wide block per CU (three quarters to all of them), 16 channels or more: 5-32 % ahead of the
+    // kernels below, whose blocks are finer than there are CUs to fill
+    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 16) {
+        const long blocks = S * (N / 128);
+        if (4 * blocks >= 3L * cu_count() && blocks <= cu_count()) return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
+    }
+    // DY = 128 with N not a multiple of 128 (tiles of 64, three real products): one to two blocks per CU, 16 channels or
+    // more: 6-22 % ahead; with 128 channels up to four per CU (12 %)
+    if (algo == 0 && logDY == 7 && N % 128 != 0 && K >= 16) {
+        const long blocks = S * (N / 64);
+        if (blocks >= cu_count() && blocks <= (K >= 128 ? 4L : 2L) * cu_count())
+            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
+    }
+    // DY = 256, N not a multiple of 128, 128 channels or more, up to four blocks of 64-channel tiles per CU: 6-8 % ahead
+    if (algo == 0 && logDY == 8 && N % 128 != 0 && K >= 128) {
+        const long blocks = S * (N / 64);
+        if (blocks > cu_count() && blocks <= 4L * cu_count()) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream, keep_y);
+    }
     if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
         return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
     if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cu_count() : (K >= 24 && items >= 128L * cu_count())))
@@ -805,7 +823,10 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
     if (algo == 8 && (logDY == 7 || logDY == 8)) return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream, keep_y);
     if (algo == 8) algo = 0;
     int pick = algo == 4 ? 2 : algo;
-    if (pick == 0) pick = (built && items <= cu_count()) ? 2 : (!long_signal ? 3 : 1);
+    // lengths 512 / 1024 with 64 channels or more, x and y streamed: the 256-thread matrix-core kernel is 7-16 % ahead of
+    // the SIMT kernel on grids of up to four blocks per CU (level or up to 10 % behind on larger ones)
+    if (pick == 0)
+        pick = (built && items <= cu_count()) ? 2 : ((!long_signal || (K >= 64 && !keep_y && items <= 4L * cu_count())) ? 3 : 1);
     // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
     // shares the spectra through LDS; level at K = 32)
     if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cu_count()))) {
