@@ -70,9 +70,9 @@ int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
     if (bs < 4) return TURBOFNO_2D_THREE_KERNEL;
     const bool big = DX == 256 && DY == 256;
     if (bs >= 8) {
-        // two exceptions measured 7-13 % behind: few images of 256 x 256, and 256 x 128 images with 64 output channels
+        // two exceptions measured 7-15 % behind: few images of 256 x 256, and rows of 128 with 64 output channels
         if (big && ((long)K + N) * bs < 768) return TURBOFNO_2D_THREE_KERNEL;
-        if (DX == 256 && DY == 128 && N == 64 && K < 128) return TURBOFNO_2D_THREE_KERNEL;
+        if (DY == 128 && N == 64 && K < 128) return TURBOFNO_2D_THREE_KERNEL;
         return TURBOFNO_2D_WHOLE_IMAGE;
     }
     if (big && ((long)K + N) * bs >= 768) return TURBOFNO_2D_WHOLE_IMAGE;
