@@ -9,8 +9,10 @@
  *
  * Conventions
  *   - All data pointers are DEVICE pointers to complex64 (interleaved float re, im). The caller owns
- *     every buffer; the library allocates nothing and never synchronises the device.
- *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Calls are asynchronous.
+ *     every buffer, including the 2D workspace and the optional exchange buffer of clustered launches;
+ *     no entry point allocates or frees memory, on the device or pinned on the host.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream). Calls are asynchronous and
+ *     never synchronise, with one documented exception: turbofno_exchange_status waits for its stream.
  *   - Return value 0 = success; otherwise a TURBOFNO_ERR_* code, with a human-readable explanation
  *     available from turbofno_last_error_string() (thread local). The library never exits the process
  *     (the reference exits from its mains via CHECK_CUDA_KERNEL, utils/utils.cuh:17-25).
@@ -33,7 +35,7 @@ extern "C" {
 #define TURBOFNO_ERR_UNSUPPORTED  2  /* transform length outside the built set                           */
 #define TURBOFNO_ERR_WORKSPACE    3  /* workspace missing or too small                                   */
 #define TURBOFNO_ERR_HIP          4  /* the HIP runtime reported a launch error                          */
-#define TURBOFNO_ERR_EXCHANGE     5  /* an earlier clustered launch on this stream gave up an inter-block wait */
+#define TURBOFNO_ERR_EXCHANGE     5  /* turbofno_exchange_status only: cluster members ran out of their wait (results valid, launches slow) */
 
 #define TURBOFNO_MODES 64
 
@@ -51,8 +53,8 @@ extern "C" {
  * M = 64 * S where S = bs*dimX signals per channel. `C` is unused by the reference kernel (its beta*C
  * term is commented out, fused_fft_cgemm_ifft_7.cuh:186-187) and may be NULL; beta is ignored.
  * Requires logDY in {7, 8, 9, 10}, M % 64 == 0, N % 64 == 0, K % 8 == 0 (utils/TurboFNO.h:2-4).
- * On small grids with K >= 64 this entry point and turbofno_layer_1d may use a library-owned exchange buffer and
- * return TURBOFNO_ERR_EXCHANGE: see "Clustered launches" below.
+ * On small grids with K >= 64 this entry point and turbofno_layer_1d use the exchange buffer of the stream when the
+ * caller has attached one: see "Clustered launches" below.
  */
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
                                   float alpha_re, float alpha_im, float beta_re, float beta_im, void* stream);
@@ -141,7 +143,8 @@ int turbofno_fused_cgemm_ifft(int logDY, long M, int N, int K, const void* A, co
  * harnesses that forbid hipMalloc. No counterpart in the reference (its mains allocate every buffer themselves,
  * fused_trunc_2D.cu:68-85). Same arguments and results as turbofno_layer_2d, without the workspace: the
  * intermediates live in a static device array of TURBOFNO_NOALLOC_SCRATCH_BYTES that every GPU the library runs on
- * holds until the process ends. The call allocates and frees nothing. Problems whose intermediates
+ * holds until the process ends. The call allocates and frees nothing, whatever the sizes and whether or not an exchange
+ * buffer is attached to the stream. `stream` must belong to the current device. Problems whose intermediates
  * (turbofno_layer_2d_workspace_bytes with the same arguments) exceed that size are refused with
  * TURBOFNO_ERR_WORKSPACE; the headline problem bs=16, 256 x 256, K=N=64 fits exactly. The first call on a device
  * resolves the array's address (make it outside any graph capture). All calls on one GPU share the one array:
@@ -165,26 +168,58 @@ int turbofno_set_1d_algo(int algo);
 int turbofno_get_1d_algo(void);
 
 /*
- * Clustered launches (no counterpart in the reference). On small grids with K >= 64 (DY = 256, N = 64 or 128, every
- * block on a CU of its own) the fused 1D layer splits the K channels of a signal set over 2 - 8 blocks, which exchange
- * partial products through a device buffer that the library owns: one per (device, stream) that has used this path,
- * 64 KiB per compute unit (16 MiB on 256 CUs), allocated on first use, never moved, and kept until the process ends. Consequences for callers:
- *   - calls on one stream are ordered and share the buffer; calls on different streams use different buffers;
- *   - the first such call on a stream allocates (and synchronises the device once); inside a stream capture that is
- *     not possible, and a kernel without the exchange runs instead. A captured launch keeps using the buffer of the
- *     stream it was captured on: do not replay it concurrently with other 1D layer calls on that stream;
- *   - every inter-block wait is bounded (default 2 s). A block that runs into the bound gives up, the launch completes
- *     with invalid output, and the NEXT 1D layer call on that stream returns TURBOFNO_ERR_EXCHANGE once, without
- *     launching. turbofno_set_exchange_wait_us changes the bound (microseconds, process-wide; 0 = give up at once,
- *     for tests of this error path).
+ * Clustered launches (no counterpart in the reference; opt-in). On small grids with K >= 64 (DY = 256, N = 64 or 128,
+ * every block on a CU of its own: the reference's large-hidden 1D shapes) the fused 1D layer can split the K channels of
+ * a signal set over 2 - 8 blocks, which exchange partial products through device memory, instead of repeating all K
+ * forward transforms in every block of a signal set. That memory is the CALLER's:
+ *   turbofno_exchange_bytes(cu)   size of an exchange buffer for a device of `cu` compute units (0 = the current
+ *                                 device): 64 KiB + 128 B per compute unit + 256 B (16.03 MiB on 256 CUs);
+ *   turbofno_exchange_attach      registers `buffer` (device memory, 256-byte aligned, at least that size) for the 1D
+ *                                 layer calls on `stream` of the current device and clears its counters with a small
+ *                                 kernel on that stream (no allocation, no synchronisation). Not inside a capture of
+ *                                 that stream. Attaching again replaces the buffer;
+ *   turbofno_exchange_detach      forgets it. Detach before freeing the buffer or destroying the stream; work already
+ *                                 enqueued (or captured into a graph) keeps using the memory until it has run.
+ * While a buffer is attached, turbofno_fused_fft_cgemm_ifft / turbofno_layer_1d on that stream (and the middle stage of
+ * the three-stage 2D paths) take the clustered kernel where it applies by size; without one they run kernels that need
+ * no exchange. Calls on one stream are ordered and share its buffer; use one buffer per stream, never one buffer on two
+ * streams. A graph captured on the stream holds the buffer's address: do not replay it concurrently with other 1D
+ * layer calls that use the same buffer.
+ * Results do not depend on the exchange working: every inter-block wait is bounded (default 2 s,
+ * turbofno_set_exchange_wait_us, process-wide; 0 = do not wait at all, for tests), and a cluster member whose wait runs
+ * out computes the other members' share itself, so the output of every launch is valid - only late. Such events are
+ * counted in the buffer:
+ *   turbofno_exchange_status      WAITS for the work enqueued on `stream`, then stores the number of members that ran
+ *                                 out of their wait since the last call in *gave_up (may be NULL) and clears it;
+ *                                 returns TURBOFNO_ERR_EXCHANGE when that number is not zero (advisory: the clustered
+ *                                 kernel does not suit the way this process shares the GPU), TURBOFNO_OK otherwise and
+ *                                 when no buffer is attached.
  */
+size_t turbofno_exchange_bytes(int compute_units);
+int turbofno_exchange_attach(void* stream, void* buffer, size_t bytes);
+int turbofno_exchange_detach(void* stream);
+int turbofno_exchange_status(void* stream, unsigned* gave_up);
 int turbofno_set_exchange_wait_us(unsigned long long microseconds);
+
+/*
+ * What the size rules choose, as plain integer functions (no GPU work; no counterpart in the reference, whose tables
+ * are indexed by log2(length) - 7 alone):
+ *   turbofno_query_2d_algo    the algorithm turbofno_layer_2d(..., algo) runs for these sizes: TURBOFNO_2D_THREE_KERNEL,
+ *                             _WHOLE_IMAGE or _ROWS_FIRST; 0 for arguments the layer would refuse.
+ *   turbofno_query_1d_kernel  the kernel behind turbofno_fused_fft_cgemm_ifft(logDY, M, N, K, ...) under the current
+ *                             turbofno_set_1d_algo selector, in that selector's numbering (1 ... 8); 0 for arguments
+ *                             the call would refuse. compute_units = 0 asks the current device (the only case that
+ *                             touches the HIP runtime), any other value answers for a device of that many compute
+ *                             units; exchange_attached says whether the stream has an exchange buffer.
+ */
+int turbofno_query_2d_algo(int bs, int DX, int DY, int K, int N, int algo);
+int turbofno_query_1d_kernel(int logDY, long M, int N, int K, int compute_units, int exchange_attached);
 
 /* Explanation of the last non-zero return value on this thread ("" if none). Never NULL. */
 const char* turbofno_last_error_string(void);
 
 /* ABI version of this header (bumped on incompatible change). */
-int turbofno_abi_version(void);
+int turbofno_abi_version(void);   /* 2: exchange buffers are caller-owned; query functions */
 
 #ifdef __cplusplus
 }

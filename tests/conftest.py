@@ -42,10 +42,21 @@ def max_rel_elementwise(a, b, floor_frac=1e-2):
 
 @pytest.fixture
 def algo_1d():
-    """sets the process-wide choice of the fused 1D kernel for one test and restores the choice by size afterwards"""
+    """sets the process-wide choice of the fused 1D kernel for one test and restores the choice by size afterwards.
+    Selector 7 (a cluster of blocks per signal set) only runs on streams with an exchange buffer: unless attach=False,
+    one is attached to torch's current stream for the rest of the test."""
     import turbofno_amd as tf
-    yield tf.set_1d_algo
+    held = []
+
+    def choose(algo, attach=True):
+        if algo == 7 and attach and not held:
+            held.append(tf.ExchangeBuffer())
+        return tf.set_1d_algo(algo)
+
+    yield choose
     tf.set_1d_algo(0)
+    for b in held:
+        b.close()
 
 
 @pytest.fixture(scope="session")

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_abi_version_and_error_string_without_gpu():
     L = tf.lib()
-    assert L.turbofno_abi_version() == 1
+    assert L.turbofno_abi_version() == 2
     assert L.turbofno_last_error_string() is not None
     # argument validation happens before any GPU call
     rc = L.turbofno_fused_fft_cgemm_ifft(8, 64, 64, 12, 1, 1, None, 1, 1.0, 0.0, 0.0, 0.0, None)

@@ -1,8 +1,11 @@
 """The clustered fused 1D kernel (small grids, K >= 64, DY = 256, N in {64, 128}): several blocks share a signal set,
-split its K channels and exchange partial products through a library-owned device buffer. Checked against the CPU
-oracle on the shapes that select each cluster size and chunk size, across repeated launches (the arrival counters are
-never reset), on two streams at once (separate buffers), from a replayed graph, and on the error path of a wait that
-gives up."""
+split its K channels and exchange partial products through a CALLER-owned device buffer that is attached to a stream.
+Checked against the CPU oracle on the shapes that select each cluster size and chunk size, across repeated launches (the
+arrival counters are never reset), on two streams at once (one buffer each), from a replayed graph, and with a wait
+bound of zero, where every member that would have to wait computes the other members' share itself: the output stays
+valid and the event is counted. Without an attached buffer the library must neither allocate nor take this kernel."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -26,6 +29,13 @@ def check(got, ref, tol, what):
     assert e2 <= tol["l2"] and em <= tol["max"] and ee <= tol["elem"], (what, e2, em, ee)
 
 
+@pytest.fixture
+def exchange():
+    """an exchange buffer attached to torch's current stream for the duration of one test"""
+    with tf.ExchangeBuffer() as ex:
+        yield ex
+
+
 # S, K, N -> cluster size / channels per member / chunk (on 256 CUs)
 SHAPES = [
     (64, 128, 128),   # the large-hidden benchmark case: 4 members x 32 channels, one chunk of 32
@@ -44,9 +54,10 @@ SHAPES = [
 
 @pytest.mark.parametrize("algo", [0, 7])
 @pytest.mark.parametrize("S,K,N", SHAPES)
-def test_cluster_against_oracle(S, K, N, algo, tol, algo_1d):
+def test_cluster_against_oracle(S, K, N, algo, tol, algo_1d, exchange):
     print("case cluster", S, K, N, "algo", algo, flush=True)
-    algo_1d(algo)
+    algo_1d(algo, attach=False)
+    assert tf.query_1d_kernel(256, S, N, K, compute_units=0, exchange_attached=True) == 7
     x, W = workloads.uniform_1d(300 + S + K + N, S, 256, K, N)
     ref = oracle.layer_1d(x, W, 0.75 - 0.5j)
     xd, Wd = dev(x), dev(W)
@@ -54,9 +65,10 @@ def test_cluster_against_oracle(S, K, N, algo, tol, algo_1d):
         y = tf.layer_1d(xd, Wd, alpha=0.75 - 0.5j)
         torch.cuda.synchronize()
         check(y, ref, tol, "cluster S=%d K=%d N=%d launch %d" % (S, K, N, rep))
+    assert exchange.status() == 0   # a grid of one block per CU on an otherwise idle GPU never runs out of its wait
 
 
-def test_cluster_matches_block_kernel_on_the_large_hidden_case(tol, algo_1d):
+def test_cluster_matches_block_kernel_on_the_large_hidden_case(tol, algo_1d, exchange):
     """bs = 64, DY = 256, K = N = 128 with the generator the benchmark uses: clustered kernel against the kernel that
     keeps a signal set inside one block (no exchange), element by element"""
     print("case cluster vs block kernel", flush=True)
@@ -64,43 +76,73 @@ def test_cluster_matches_block_kernel_on_the_large_hidden_case(tol, algo_1d):
     xd, Wd = dev(x), dev(W)
     algo_1d(2)
     ref = tf.layer_1d(xd, Wd).cpu().numpy()
-    algo_1d(7)
+    algo_1d(7, attach=False)
     check(tf.layer_1d(xd, Wd), ref, tol, "cluster vs block kernel")
+
+
+def test_without_a_buffer_nothing_is_allocated_and_another_kernel_runs(tol, algo_1d):
+    """no exchange buffer attached: the choice by size (and the forced selector 7) fall back on the kernel that splits
+    K inside one block, and the call leaves the free device memory exactly as it found it"""
+    print("case no buffer", flush=True)
+    S, K, N = 64, 128, 128
+    assert tf.query_1d_kernel(256, S, N, K, compute_units=0, exchange_attached=False) == 6
+    x, W = workloads.uniform_1d(41, S, 256, K, N)
+    ref = oracle.layer_1d(x, W, 1.0)
+    xd, Wd = dev(x), dev(W)
+    y = torch.empty((N, S, 256), dtype=torch.complex64, device="cuda")
+    tf.layer_1d(xd, Wd, y=y)                    # the HIP runtime's own first-launch work for this kernel happens here
+    side = torch.cuda.Stream()                  # a stream the library has never seen;
+    with torch.cuda.stream(side):
+        y.zero_()                               # ... and the runtime's per-stream set-up here
+    torch.cuda.synchronize()
+    for algo in (0, 7):
+        algo_1d(algo, attach=False)
+        free_before = torch.cuda.mem_get_info()[0]
+        with torch.cuda.stream(side):
+            tf.layer_1d(xd, Wd, y=y)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "the 1D layer call changed the free device memory"
+        check(y, ref, tol, "no buffer, selector %d" % algo)
 
 
 def test_cluster_on_two_streams(tol, algo_1d):
     """launches on two streams overlap on the GPU; each stream has its own exchange buffer"""
     print("case cluster two streams", flush=True)
-    algo_1d(7)
+    algo_1d(7, attach=False)
     S, K, N = 24, 128, 128
     probs = []
     for i in range(2):
         x, W = workloads.uniform_1d(900 + i, S, 256, K, N)
         probs.append((dev(x), dev(W), oracle.layer_1d(x, W, 1.0), torch.empty((N, S, 256), dtype=torch.complex64, device="cuda")))
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    buffers = [tf.ExchangeBuffer(stream=st) for st in streams]
     torch.cuda.synchronize()
-    for _ in range(20):
-        for (xd, Wd, _, y), st in zip(probs, streams):
-            with torch.cuda.stream(st):
-                tf.layer_1d(xd, Wd, y=y)
-    torch.cuda.synchronize()
+    try:
+        for _ in range(20):
+            for (xd, Wd, _, y), st in zip(probs, streams):
+                with torch.cuda.stream(st):
+                    tf.layer_1d(xd, Wd, y=y)
+        torch.cuda.synchronize()
+    finally:
+        for b in buffers:
+            b.close()
     for i, (_, _, ref, y) in enumerate(probs):
         check(y, ref, tol, "cluster stream %d" % i)
 
 
 def test_cluster_in_a_replayed_graph(tol, algo_1d):
-    """captured after a first eager call (which allocates the stream's buffer); every replay is checked, with eager
-    launches on the same stream in between"""
+    """the buffer is attached before the capture; every replay is checked, with eager launches on the same stream in
+    between (they share the stream's buffer and its counters)"""
     print("case cluster graph", flush=True)
-    algo_1d(7)
+    algo_1d(7, attach=False)
     S, K, N = 64, 128, 128
     x, W = workloads.uniform_1d(77, S, 256, K, N)
     ref = oracle.layer_1d(x, W, 1.0)
     xd, Wd = dev(x), dev(W)
     y = torch.empty((N, S, 256), dtype=torch.complex64, device="cuda")
     side = torch.cuda.Stream()
-    with torch.cuda.stream(side):
-        tf.layer_1d(xd, Wd, y=y)                    # allocates the exchange buffer of this stream
+    with torch.cuda.stream(side), tf.ExchangeBuffer(stream=side):
+        tf.layer_1d(xd, Wd, y=y)
         side.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
@@ -115,25 +157,46 @@ def test_cluster_in_a_replayed_graph(tol, algo_1d):
             check(y2, ref, tol, "cluster eager after replay %d" % rep)
 
 
-def test_cluster_wait_that_gives_up_is_reported(tol, algo_1d):
-    """with a wait bound of zero every block that has to wait gives up (all kernels still run to completion); the next
-    call on the stream reports it once, the one after that works again"""
-    print("case cluster gives up", flush=True)
-    algo_1d(7)
-    S, K, N = 64, 128, 128
-    x, W = workloads.uniform_1d(78, S, 256, K, N)
+@pytest.mark.parametrize("S,K,N,P", [(64, 128, 128, 4), (5, 192, 64, 8), (128, 64, 64, 2)])
+def test_cluster_member_that_runs_out_of_its_wait_still_delivers(S, K, N, P, tol, algo_1d, exchange):
+    """with a wait bound of zero every member that finds its cluster incomplete computes the other members' share
+    itself (all kernels run to completion): the output is valid, the event is counted once, and the following
+    launches use the exchange again"""
+    print("case cluster runs out of its wait", S, K, N, flush=True)
+    algo_1d(7, attach=False)
+    x, W = workloads.uniform_1d(78 + S, S, 256, K, N)
+    ref = oracle.layer_1d(x, W, 0.5 + 0.25j)
     xd, Wd = dev(x), dev(W)
-    tf.layer_1d(xd, Wd)
-    torch.cuda.synchronize()
+    tf.layer_1d(xd, Wd, alpha=0.5 + 0.25j)
+    assert exchange.status() == 0
     tf.set_exchange_wait_us(0)
     try:
-        tf.layer_1d(xd, Wd)                         # output invalid
+        y = tf.layer_1d(xd, Wd, alpha=0.5 + 0.25j)
         torch.cuda.synchronize()
     finally:
         tf.set_exchange_wait_us(2_000_000)
-    with pytest.raises(tf.TurboFNOError) as err:
-        tf.layer_1d(xd, Wd)
-    assert err.value.code == 5, err.value
-    y = tf.layer_1d(xd, Wd)
+    check(y, ref, tol, "cluster without waiting")
+    n = ctypes.c_uint(0)
+    rc = tf.lib().turbofno_exchange_status(torch.cuda.current_stream().cuda_stream, ctypes.byref(n))
+    assert rc == 5 and n.value == S * (P - 1), (rc, n.value)            # every member but the last of each cluster
+    assert b"valid" in tf.lib().turbofno_last_error_string()
+    assert exchange.status() == 0                                       # reported once
+    y = tf.layer_1d(xd, Wd, alpha=0.5 + 0.25j)
     torch.cuda.synchronize()
-    check(y, oracle.layer_1d(x, W, 1.0), tol, "cluster after a reported give-up")
+    check(y, ref, tol, "cluster after a counted event")
+    assert exchange.status() == 0
+
+
+def test_attach_refuses_a_buffer_that_is_too_small_or_misaligned():
+    L = tf.lib()
+    need = tf.exchange_bytes(0)
+    assert need == tf.exchange_bytes(torch.cuda.get_device_properties(0).multi_processor_count)
+    buf = torch.empty(need + 512, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    assert L.turbofno_exchange_attach(st, buf.data_ptr(), need - 1) == 3
+    assert L.turbofno_exchange_attach(st, buf.data_ptr() + 8, need) == 3
+    assert L.turbofno_exchange_attach(st, None, need) == 1
+    assert L.turbofno_exchange_attach(st, buf.data_ptr(), need) == 0
+    assert L.turbofno_exchange_detach(st) == 0
+    assert L.turbofno_exchange_detach(st) == 0                          # nothing attached: still fine
+    torch.cuda.synchronize()

@@ -47,9 +47,7 @@ def test_layer_1d_in_a_graph(K):
     W = torch.from_numpy(workloads.smooth_1d(950, bs, DY, K, N)[1]).cuda()
     x = xs[0].clone()
     y = torch.empty((N, bs, DY), dtype=torch.complex64, device="cuda")
-    # the warm-up runs on the stream that is captured afterwards: at K = 128 the clustered kernel is chosen, whose
-    # exchange buffer belongs to a stream and cannot be created during a capture (a kernel without the exchange would
-    # be captured instead, and the bit-for-bit comparison below would compare two different kernels)
+    # warm-up on the stream that is captured afterwards (raises the kernels' dynamic-LDS limits outside the capture)
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         tf.layer_1d(x, W, y=y)

@@ -57,6 +57,34 @@ def test_driver_result_lines(tmp_path):
     assert got == [(1, 128, 128, 64, 8), (1, 128, 128, 64, 16), (1, 256, 128, 64, 8), (1, 256, 128, 64, 16)], lines
 
 
+def test_driver_refuses_malformed_arguments_before_touching_the_gpu():
+    """five positional arguments that are not positive integers end the run with a message (no HIP call has happened
+    yet, so this runs without a GPU)"""
+    for v in "AD":
+        exe = os.path.join(ROOT, "bin", f"TurboFNO_1D_{v}")
+        assert os.path.exists(exe), "build the drivers with make -C turbofno_amd/host"
+        for bad in (["4", "1", "12x", "64", "16"], ["0", "1", "128", "64", "16"], ["4", "1", "128", "", "16"],
+                    ["4", "1", "128", "64", "99999999999"]):
+            r = subprocess.run([exe] + bad, capture_output=True, text=True, timeout=100)
+            assert r.returncode == 1 and "is not a positive integer" in r.stderr and r.stdout == "", (bad, r)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", "ABCD")
+def test_driver_skips_lengths_without_a_kernel(variant, tmp_path):
+    """a length that is not 128, 256, 512 or 1024 has no kernel-table entry: every variant prints why and skips the
+    problem instead of running a kernel of a neighbouring length on its buffers"""
+    cfg = str(tmp_path / "odd_2d.txt")
+    with open(cfg, "w") as f:
+        f.write("bs_list = 1\nDX_list = 128 200\nDY_list = 128 96\nN_list = 64 96\nK_list = 8")
+    exe = os.path.join(ROOT, "bin", f"TurboFNO_2D_{variant}")
+    r = subprocess.run([exe, cfg], check=True, capture_output=True, text=True, timeout=100)
+    lines = r.stdout.splitlines()
+    got = [tuple(int(v) for v in re.findall(r"=(\d+)", ln)[:5]) for ln in lines]
+    assert got == [(1, 128, 128, 64, 8)], (lines, r.stderr)
+    assert r.stderr.count("problem skipped") == 7, r.stderr
+
+
 def test_seeded_input_generators(tmp_path):
     """the C++ generators of the benchmark configurations' inputs: ranges, unit variance, smoothness, reproducibility"""
     exe = str(tmp_path / "inputs_check")

@@ -7,8 +7,10 @@ library fallback: if the shared library is missing, importing `turbofno_amd.api`
 """
 from .api import (  # noqa: F401
     MODES,
+    ExchangeBuffer,
     TurboFNOError,
     cgemm,
+    exchange_bytes,
     fft2d_trunc,
     ifft2d_pad,
     fft_stride,
@@ -24,8 +26,10 @@ from .api import (  # noqa: F401
     layer_2d_workspace_bytes,
     lib,
     library_path,
+    query_1d_kernel,
+    query_2d_algo,
     set_1d_algo,
     set_exchange_wait_us,
 )
 
-ALGO_AUTO, ALGO_THREE_KERNEL, ALGO_WHOLE_IMAGE = 0, 1, 2
+ALGO_AUTO, ALGO_THREE_KERNEL, ALGO_WHOLE_IMAGE, ALGO_ROWS_FIRST = 0, 1, 2, 3

@@ -55,6 +55,18 @@ def lib():
         L.turbofno_set_exchange_wait_us.argtypes = [ctypes.c_ulonglong]
         L.turbofno_set_exchange_wait_us.restype = i
         L.turbofno_get_1d_algo.restype = i
+        L.turbofno_exchange_bytes.argtypes = [i]
+        L.turbofno_exchange_bytes.restype = sz
+        L.turbofno_exchange_attach.argtypes = [vp, vp, sz]
+        L.turbofno_exchange_attach.restype = i
+        L.turbofno_exchange_detach.argtypes = [vp]
+        L.turbofno_exchange_detach.restype = i
+        L.turbofno_exchange_status.argtypes = [vp, ctypes.POINTER(ctypes.c_uint)]
+        L.turbofno_exchange_status.restype = i
+        L.turbofno_query_2d_algo.argtypes = [i, i, i, i, i, i]
+        L.turbofno_query_2d_algo.restype = i
+        L.turbofno_query_1d_kernel.argtypes = [i, l, i, i, i, i]
+        L.turbofno_query_1d_kernel.restype = i
         L.turbofno_last_error_string.restype = ctypes.c_char_p
         L.turbofno_abi_version.restype = i
         for name in ("turbofno_fused_fft_cgemm_ifft", "turbofno_fft_stride", "turbofno_ifft_stride",
@@ -115,6 +127,53 @@ def set_1d_algo(algo):
 def set_exchange_wait_us(microseconds):
     """Bound of the inter-block waits of the clustered 1D kernel (include/turbofno.h); 0 = give up at once."""
     _check(lib().turbofno_set_exchange_wait_us(int(microseconds)))
+
+
+def exchange_bytes(compute_units=0):
+    """Size of an exchange buffer for clustered 1D launches (0 = the current device; needs a GPU then)."""
+    return int(lib().turbofno_exchange_bytes(int(compute_units)))
+
+
+class ExchangeBuffer:
+    """A caller-owned exchange buffer attached to torch's current stream (turbofno_exchange_attach); detaches on
+    close() / at the end of a `with` block. The tensor lives as long as this object."""
+
+    def __init__(self, stream=None):
+        self._stream = torch.cuda.current_stream() if stream is None else stream
+        self.buffer = torch.empty(exchange_bytes(0), dtype=torch.uint8, device="cuda")
+        _check(lib().turbofno_exchange_attach(self._stream.cuda_stream, self.buffer.data_ptr(), self.buffer.numel()))
+
+    def status(self):
+        """waits for the stream; number of cluster members that ran out of their wait since the last call"""
+        n = ctypes.c_uint(0)
+        rc = lib().turbofno_exchange_status(self._stream.cuda_stream, ctypes.byref(n))
+        if rc not in (0, 5):
+            _check(rc)
+        return int(n.value)
+
+    def close(self):
+        if self.buffer is not None:
+            _check(lib().turbofno_exchange_detach(self._stream.cuda_stream))
+            self._stream.synchronize()          # enqueued work may still use the memory
+            self.buffer = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+        return False
+
+
+def query_2d_algo(bs, DX, DY, K, N, algo=0):
+    """The algorithm layer_2d runs for these sizes (1 three kernels, 2 whole image, 3 rows first; 0 = refused)."""
+    return int(lib().turbofno_query_2d_algo(bs, DX, DY, K, N, algo))
+
+
+def query_1d_kernel(DY, S, N, K, compute_units=256, exchange_attached=False):
+    """The fused 1D kernel (numbering of set_1d_algo, 1 ... 8) for S signals per channel; 0 = refused. With an explicit
+    compute_units this is pure arithmetic (no GPU needed)."""
+    return int(lib().turbofno_query_1d_kernel(_log2(DY), MODES * S, N, K, int(compute_units), 1 if exchange_attached else 0))
 
 
 def fused_fft_cgemm_ifft(M, N, K, x, W, y, alpha=1.0 + 0j, beta=0j, C=None):

@@ -22,9 +22,6 @@ int fail(int code, const char* fmt, ...)
 int hip_status(hipError_t e, const char* what)
 {
     if (e == hipSuccess) return TURBOFNO_OK;
-    if (e == hipErrorLaunchTimeOut)         // reported by the clustered 1D launcher, never by a launch itself
-        return fail(TURBOFNO_ERR_EXCHANGE, "%s: a block of an earlier clustered launch on this stream gave up waiting for its cluster; "
-                                           "that launch's output is invalid", what);
     return fail(TURBOFNO_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
@@ -84,7 +81,7 @@ int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 
 extern "C" {
 
-int turbofno_abi_version(void) { return 1; }
+int turbofno_abi_version(void) { return 2; }
 
 const char* turbofno_last_error_string(void) { return g_err; }
 
@@ -110,6 +107,55 @@ int turbofno_set_exchange_wait_us(unsigned long long microseconds)
 {
     tfno::set_cluster_wait_ticks(microseconds > (~0ull) / 100 ? ~0ull : microseconds * 100);   // 100 MHz wall clock
     return TURBOFNO_OK;
+}
+
+size_t turbofno_exchange_bytes(int compute_units) { return tfno::exchange_bytes(compute_units); }
+
+int turbofno_exchange_attach(void* stream, void* buffer, size_t bytes)
+{
+    if (!buffer) return fail(TURBOFNO_ERR_INVALID_ARG, "buffer must be a non-null device pointer (turbofno_exchange_detach forgets a buffer)");
+    const hipError_t e = tfno::exchange_attach((hipStream_t)stream, buffer, bytes);
+    if (e == hipErrorInvalidValue)
+        return fail(TURBOFNO_ERR_WORKSPACE, "exchange buffer must be 256-byte aligned and hold turbofno_exchange_bytes(0) = %zu bytes (%zu given)",
+                    tfno::exchange_bytes(0), bytes);
+    if (e == hipErrorStreamCaptureUnsupported)
+        return fail(TURBOFNO_ERR_INVALID_ARG, "the stream is being captured: attach the exchange buffer before the capture begins");
+    return hip_status(e, "exchange_attach");
+}
+
+int turbofno_exchange_detach(void* stream) { return hip_status(tfno::exchange_attach((hipStream_t)stream, nullptr, 0), "exchange_detach"); }
+
+int turbofno_exchange_status(void* stream, unsigned* gave_up)
+{
+    unsigned count = 0;
+    const hipError_t e = tfno::exchange_gave_up((hipStream_t)stream, &count);
+    if (e == hipErrorNotReady) {                                 // nothing attached: nothing can have waited
+        if (gave_up) *gave_up = 0;
+        return TURBOFNO_OK;
+    }
+    if (int rc = hip_status(e, "exchange_status")) return rc;
+    if (gave_up) *gave_up = count;
+    if (count)
+        return fail(TURBOFNO_ERR_EXCHANGE, "%u cluster member(s) on this stream ran out of their wait and computed the other members' share "
+                                           "themselves (results are valid; the launches were slow)", count);
+    return TURBOFNO_OK;
+}
+
+int turbofno_query_1d_kernel(int logDY, long M, int N, int K, int compute_units, int exchange_attached)
+{
+    if (check_gemm_dims(M, N, K) || !length_built(logDY)) return 0;
+    const long cus = compute_units > 0 ? compute_units : tfno::cu_count();
+    return tfno::pick_fused_1d_kernel(logDY, M / 64, N, K, algo_1d(), false, cus, exchange_attached != 0);
+}
+
+int turbofno_query_2d_algo(int bs, int DX, int DY, int K, int N, int algo)
+{
+    if (bs <= 0 || K <= 0 || N <= 0 || K % 8 || N % 64) return 0;
+    const int logDX = log2_exact(DX), logDY = log2_exact(DY);
+    if (!length_built(logDX) || !length_built(logDY)) return 0;
+    if (algo < TURBOFNO_2D_AUTO || algo > TURBOFNO_2D_ROWS_FIRST) return 0;
+    if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256)) return 0;
+    return pick_algo(bs, DX, DY, K, N, algo);
 }
 
 int turbofno_fused_fft_cgemm_ifft(int logDY, long M, int N, int K, const void* x, const void* W, void* C, void* y,
@@ -307,10 +353,18 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
 static __device__ __align__(256) unsigned char scratch[TURBOFNO_NOALLOC_SCRATCH_BYTES];
 static std::atomic<void*> g_scratch_ptr[64];
 
-static int scratch_of_current_device(void** out)
+static int scratch_of_current_device(void* stream, void** out)
 {
     int dev = 0;
     if (int rc = hip_status(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    // The kernels run on the stream's device and must get THAT device's copy of the array. A launch on a stream of
+    // another device than the current one is refused rather than resolved behind the caller's back.
+    if (stream && (hipStream_t)stream != hipStreamPerThread && (hipStream_t)stream != hipStreamLegacy) {
+        int sdev = dev;
+        if (int rc = hip_status(hipStreamGetDevice((hipStream_t)stream, &sdev), "hipStreamGetDevice")) return rc;
+        if (sdev != dev)
+            return fail(TURBOFNO_ERR_INVALID_ARG, "the stream belongs to device %d, the current device is %d: make the stream's device current", sdev, dev);
+    }
     if (dev < 0 || dev >= 64) return fail(TURBOFNO_ERR_UNSUPPORTED, "device ordinal %d: the static scratch is tracked for ordinals below 64", dev);
     void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!p) {
@@ -334,7 +388,7 @@ int turbofno_layer_2d_noalloc(int bs, int DX, int DY, int K, int N, const void* 
                         "a workspace, or split the batch", need, (size_t)TURBOFNO_NOALLOC_SCRATCH_BYTES);
     }
     void* ptr = nullptr;
-    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    if (int rc = scratch_of_current_device(stream, &ptr)) return rc;
     return layer_2d_on(bs, DX, DY, K, N, x, W, y, alpha_re, alpha_im, ptr, (size_t)TURBOFNO_NOALLOC_SCRATCH_BYTES,
                        "static scratch", algo, stream);
 }

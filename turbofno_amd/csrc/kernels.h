@@ -83,17 +83,27 @@ inline hipError_t allow_dynamic_lds(const void* kernel, size_t bytes, std::atomi
 }
 
 // 1D fused layer / Y stage of the three-kernel 2D pipeline. S = number of signals per channel.
-// algo: 0 = chosen by size, 1 = SIMT contraction, 2 / 3 = contraction on the matrix cores (512- / 256-thread blocks).
+// algo: 0 = chosen by size, 1 ... 8 = one of the kernels below (include/turbofno.h, turbofno_set_1d_algo).
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream, bool y_is_reread = false);
+// The kernel that call runs (the selector values 1 ... 8), from the sizes alone.
+enum {
+    kFused1dSimt = 1, kFused1dMfma512 = 2, kFused1dMfma256 = 3, kFused1dMfma512Tile32 = 4, kFused1dWave = 5,
+    kFused1dSplit = 6, kFused1dCluster = 7, kFused1dWide = 8
+};
+int pick_fused_1d_kernel(int logDY, long S, int N, int K, int algo, bool keep_y, long cus, bool exchange_attached);
 
-// Cluster variant of the fused 1D layer (layer1d_cluster.hip): cluster size for a problem (0 = not applicable), the
-// launch (hipErrorNotReady when its exchange buffer cannot be provided), and the bound of its inter-block waits in
-// ticks of the 100 MHz wall clock.
-int cluster_size_1d(int logDY, long S, int N, int K);
+// Cluster variant of the fused 1D layer (layer1d_cluster.hip): cluster size for a problem on `cus` compute units (0 = not
+// applicable), the launch (hipErrorNotReady when no exchange buffer is attached to the stream), the bound of its
+// inter-block waits in ticks of the 100 MHz wall clock, and the registry of caller-owned exchange buffers.
+int cluster_size_1d(int logDY, long S, int N, int K, long cus);
 hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
                                 hipStream_t stream);
 void set_cluster_wait_ticks(unsigned long long ticks);
+size_t exchange_bytes(long cus);                                    // cus <= 0: the current device
+hipError_t exchange_attach(hipStream_t stream, void* buffer, size_t bytes);   // null buffer: detach
+bool exchange_attached(hipStream_t stream);
+hipError_t exchange_gave_up(hipStream_t stream, unsigned* count);   // waits for the stream
 
 // Large grids, DY = 128 / 256 (layer1d_wide.hip): one block per (signal set, 128 or 64 output channels), three-real-product
 // contraction.

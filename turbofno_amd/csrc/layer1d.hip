@@ -745,91 +745,109 @@ static hipError_t launch_fused_wave(long S, int N, int K, const float2* x, const
     return hipGetLastError();
 }
 
+// Which fused 1D kernel runs for a problem: pure arithmetic on the sizes, the selector `algo`, the number of compute
+// units and whether the stream has an exchange buffer attached (no device call), so that callers and tests can ask.
 // algo: 0 = by size, 1 = SIMT kernel, 2 = matrix cores with 512-thread blocks, 3 = matrix cores with 256-thread blocks,
 // 4 = as 2 with 32-channel output tiles, 5 = matrix cores, one wavefront per (signal set, output tile),
 // 6 = matrix cores, the eight waves of a block split the K channels of one item (DY = 256),
 // 7 = matrix cores, a cluster of blocks splits the K channels of one signal set (DY = 256, N = 64 / 128, small grids),
 // 8 = matrix cores, 256-thread blocks with tiles of 128 output channels, three real products per complex one (DY = 256)
+// The return value uses the same numbers (1 ... 8). A selector value that a kernel is not built for falls back to the
+// choice by size.
+//
+// By size (measured on MI355X):
+//  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
+//    every K, even K = 8 where most of a chunk is padding;
+//  * grids of several items per SIMD: one wavefront per item (no barriers, nothing staged through LDS). At DY = 128
+//    it is ahead from two (K <= 16), four (K < 128) or eight items per CU; at DY = 256, where the block kernels are
+//    closer to what the access pattern allows, for K >= 128 (2-8 % from eight items per CU) and, K >= 24, on the
+//    very largest grids (4-6 % from 128 items per CU); below that the 256-thread block kernel is level or up to
+//    13 % ahead;
+//  * otherwise: matrix cores, 256-thread blocks, two or three per CU, for every K - measured 5-27 % ahead of the
+//    SIMT kernel on grids of 1 to 12 items per CU also for K < 32, where most of a chunk is padding (lengths
+//    512 / 1024: a tie within a few percent for every K, the SIMT kernel stays; on small grids the 512-thread
+//    kernel is 30-40 % ahead there too).
+int pick_fused_1d_kernel(int logDY, long S, int N, int K, int algo, bool keep_y, long cus, bool exchange_attached)
+{
+    const bool built = logDY >= 7 && logDY <= 10;
+    const bool long_signal = logDY >= 9;            // 512 / 1024: on large grids the block kernels tie with the SIMT kernel
+    const long items = S * (N / 64);
+    if (algo == 5 && (logDY == 7 || logDY == 8)) return kFused1dWave;
+    // N a multiple of 128, DY = 256, K >= 16: blocks with tiles of 128 output channels (every input channel transformed
+    // once per signal set, three real products per complex one): 5-20 % ahead of the kernels below on every grid that
+    // fills its two slots per CU reasonably evenly (measured from 400 blocks up; with a last round under three quarters
+    // full the 64-channel kernels, with their finer blocks, are ahead)
+    if (algo == 0 && logDY == 8 && N % 128 == 0 && K >= 16) {
+        const long blocks = S * (N / 128), slots = 2L * cus, rounds = (blocks + slots - 1) / slots;
+        if (blocks > cus && 4 * blocks >= 3 * rounds * slots) return kFused1dWide;
+    }
+    // the same at DY = 128 for K >= 64 (3-21 % ahead up to 64 blocks per CU; with fewer channels, or on the very largest
+    // grids, the one-wavefront kernel below is level or ahead)
+    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 64) {
+        const long blocks = S * (N / 128), slots = 2L * cus, rounds = (blocks + slots - 1) / slots;
+        if (blocks > cus && blocks <= 64L * cus && 4 * blocks >= 3 * rounds * slots) return kFused1dWide;
+    }
+    // DY = 128, about one wide block per CU (three quarters to all of them), 16 channels or more: 5-32 % ahead of the
+    // kernels below, whose blocks are finer than there are CUs to fill
+    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 16) {
+        const long blocks = S * (N / 128);
+        if (4 * blocks >= 3L * cus && blocks <= cus) return kFused1dWide;
+    }
+    // DY = 128 with N not a multiple of 128 (tiles of 64, three real products): one to two blocks per CU, 16 channels or
+    // more: 6-22 % ahead; with 128 channels up to four per CU (12 %)
+    if (algo == 0 && logDY == 7 && N % 128 != 0 && K >= 16) {
+        const long blocks = S * (N / 64);
+        if (blocks >= cus && blocks <= (K >= 128 ? 4L : 2L) * cus) return kFused1dWide;
+    }
+    // DY = 256, N not a multiple of 128, 128 channels or more, up to four blocks of 64-channel tiles per CU: 6-8 % ahead
+    if (algo == 0 && logDY == 8 && N % 128 != 0 && K >= 128) {
+        const long blocks = S * (N / 64);
+        if (blocks > cus && blocks <= 4L * cus) return kFused1dWide;
+    }
+    if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * cus) return kFused1dWave;
+    if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cus : (K >= 24 && items >= 128L * cus))) return kFused1dWave;
+    // small grids, 64 channels or more, N = 64 / 128: a cluster of blocks per signal set, no forward transform twice.
+    // Only for streams that have an exchange buffer attached; without one the kernels below take over.
+    if (algo == 7 || (algo == 0 && logDY == 8 && K >= 64)) {
+        if (exchange_attached && cluster_size_1d(logDY, S, N, K, cus) > 0) return kFused1dCluster;
+        if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
+    }
+    if (algo == 8 && (logDY == 7 || logDY == 8)) return kFused1dWide;
+    if (algo == 8) algo = 0;
+    int pick = algo == 4 ? 2 : algo;
+    // lengths 512 / 1024 with 64 channels or more, x and y streamed: the 256-thread matrix-core kernel is 7-16 % ahead of
+    // the SIMT kernel on grids of up to four blocks per CU (level or up to 10 % behind on larger ones)
+    if (pick == 0)
+        pick = (built && items <= cus) ? 2 : ((!long_signal || (K >= 64 && !keep_y && items <= 4L * cus)) ? 3 : 1);
+    // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
+    // shares the spectra through LDS; level at K = 32)
+    if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cus))) return kFused1dSplit;
+    // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
+    if (pick == 2 && (logDY == 7 || logDY == 8) && (algo == 4 || (algo == 0 && S * (N / 32) <= cus))) return kFused1dMfma512Tile32;
+    if (pick == 2 && built) return kFused1dMfma512;
+    if (pick == 3 && built) return kFused1dMfma256;
+    return kFused1dSimt;
+}
+
 hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* y,
                                        float2 alpha, int algo, hipStream_t stream, bool y_is_reread)
 {
     // y_is_reread (Y stage of the three-kernel 2D pipeline): the block kernels and the SIMT kernel then leave y in the
     // caches instead of streaming it past them; the other kernels ignore it
     const int keep_y = y_is_reread ? 1 : 0;
-    // by size (measured on MI355X):
-    //  * while every block has a CU to itself: matrix cores, 8 waves per block - the shortest chain of latencies for
-    //    every K, even K = 8 where most of a chunk is padding;
-    //  * grids of several items per SIMD: one wavefront per item (no barriers, nothing staged through LDS). At DY = 128
-    //    it is ahead from two (K <= 16), four (K < 128) or eight items per CU; at DY = 256, where the block kernels are
-    //    closer to what the access pattern allows, for K >= 128 (2-8 % from eight items per CU) and, K >= 24, on the
-    //    very largest grids (4-6 % from 128 items per CU); below that the 256-thread block kernel is level or up to
-    //    13 % ahead;
-    //  * otherwise: matrix cores, 256-thread blocks, two or three per CU, for every K - measured 5-27 % ahead of the
-    //    SIMT kernel on grids of 1 to 12 items per CU also for K < 32, where most of a chunk is padding (lengths
-    //    512 / 1024: a tie within a few percent for every K, the SIMT kernel stays; on small grids the 512-thread
-    //    kernel is 30-40 % ahead there too).
-    const bool built = logDY >= 7 && logDY <= 10;
-    const bool long_signal = logDY >= 9;            // 512 / 1024: on large grids the block kernels tie with the SIMT kernel
-    const long items = S * (N / 64);
-    if (algo == 5 && logDY == 8) return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (algo == 5 && logDY == 7) return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
-    // N a multiple of 128, DY = 256, K >= 16: blocks with tiles of 128 output channels (every input channel transformed
-    // once per signal set, three real products per complex one): 5-20 % ahead of the kernels below on every grid that
-    // fills its two slots per CU reasonably evenly (measured from 400 blocks up; with a last round under three quarters
-    // full the 64-channel kernels, with their finer blocks, are ahead)
-    if (algo == 0 && logDY == 8 && N % 128 == 0 && K >= 16) {
-        const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
-        if (blocks > cu_count() && 4 * blocks >= 3 * rounds * slots) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream, keep_y);
+    const long cus = cu_count();
+    int kernel = pick_fused_1d_kernel(logDY, S, N, K, algo, y_is_reread, cus, exchange_attached(stream));
+    if (kernel == kFused1dCluster) {
+        const hipError_t e = launch_fused_cluster(S, N, K, cluster_size_1d(logDY, S, N, K, cus), x, W, y, alpha, stream);
+        if (e != hipErrorNotReady) return e;
+        kernel = pick_fused_1d_kernel(logDY, S, N, K, algo, y_is_reread, cus, false);    // detached in between
     }
-    // the same at DY = 128 for K >= 64 (3-21 % ahead up to 64 blocks per CU; with fewer channels, or on the very largest
-    // grids, the one-wavefront kernel below is level or ahead)
-    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 64) {
-        const long blocks = S * (N / 128), slots = 2L * cu_count(), rounds = (blocks + slots - 1) / slots;
-        if (blocks > cu_count() && blocks <= 64L * cu_count() && 4 * blocks >= 3 * rounds * slots)
-            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
-    }
-    // DY = 128, about one wide block per CU (three quarters to all of them), 16 channels or more: 5-32 % ahead of the
-    // kernels below, whose blocks are finer than there are CUs to fill
-    if (algo == 0 && logDY == 7 && N % 128 == 0 && K >= 16) {
-        const long blocks = S * (N / 128);
-        if (4 * blocks >= 3L * cu_count() && blocks <= cu_count()) return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
-    }
-    // DY = 128 with N not a multiple of 128 (tiles of 64, three real products): one to two blocks per CU, 16 channels or
-    // more: 6-22 % ahead; with 128 channels up to four per CU (12 %)
-    if (algo == 0 && logDY == 7 && N % 128 != 0 && K >= 16) {
-        const long blocks = S * (N / 64);
-        if (blocks >= cu_count() && blocks <= (K >= 128 ? 4L : 2L) * cu_count())
-            return launch_fused_wide(7, S, N, K, x, W, y, alpha, stream, keep_y);
-    }
-    // DY = 256, N not a multiple of 128, 128 channels or more, up to four blocks of 64-channel tiles per CU: 6-8 % ahead
-    if (algo == 0 && logDY == 8 && N % 128 != 0 && K >= 128) {
-        const long blocks = S * (N / 64);
-        if (blocks > cu_count() && blocks <= 4L * cu_count()) return launch_fused_wide(8, S, N, K, x, W, y, alpha, stream, keep_y);
-    }
-    if (algo == 0 && logDY == 7 && items >= (K <= 16 ? 2 : (K < 128 ? 4 : 8)) * (long)cu_count())
-        return launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (algo == 0 && logDY == 8 && (K >= 128 ? items >= 8L * cu_count() : (K >= 24 && items >= 128L * cu_count())))
-        return launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream, keep_y);
-    // small grids, 64 channels or more, N = 64 / 128: a cluster of blocks per signal set, no forward transform twice.
-    // Without its exchange buffer (first use inside a stream capture, out of memory) the kernels below take over.
-    if (algo == 7 || (algo == 0 && logDY == 8 && K >= 64)) {
-        const int P = cluster_size_1d(logDY, S, N, K);
-        if (P > 0) {
-            const hipError_t e = launch_fused_cluster(S, N, K, P, x, W, y, alpha, stream);
-            if (e != hipErrorNotReady) return e;
-        }
-        if (algo == 7) algo = 0;                                // not applicable here: by size, as for every other value
-    }
-    if (algo == 8 && (logDY == 7 || logDY == 8)) return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream, keep_y);
-    if (algo == 8) algo = 0;
-    int pick = algo == 4 ? 2 : algo;
-    // lengths 512 / 1024 with 64 channels or more, x and y streamed: the 256-thread matrix-core kernel is 7-16 % ahead of
-    // the SIMT kernel on grids of up to four blocks per CU (level or up to 10 % behind on larger ones)
-    if (pick == 0)
-        pick = (built && items <= cu_count()) ? 2 : ((!long_signal || (K >= 64 && !keep_y && items <= 4L * cu_count())) ? 3 : 1);
-    // small grids, 64 channels or more: eight waves split the K channels of one item (10-16 % ahead of the kernel that
-    // shares the spectra through LDS; level at K = 32)
-    if (logDY == 8 && (algo == 6 || (algo == 0 && K >= 64 && S * (N / SPLIT_NT) <= cu_count()))) {
+    switch (kernel) {
+    case kFused1dWave:
+        return logDY == 8 ? launch_fused_wave<8>(S, N, K, x, W, y, alpha, stream, keep_y)
+                          : launch_fused_wave<7>(S, N, K, x, W, y, alpha, stream, keep_y);
+    case kFused1dWide: return launch_fused_wide(logDY, S, N, K, x, W, y, alpha, stream, keep_y);
+    case kFused1dSplit: {
         static std::atomic<unsigned long long> served;
         if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(fused_fft_mfma_ifft_split_kernel), SPLIT_LDS, served);
             e != hipSuccess)
@@ -839,20 +857,25 @@ hipError_t launch_fused_fft_cgemm_ifft(int logDY, long S, int N, int K, const fl
                            (int)S, N, K, x, W, y, alpha);
         return hipGetLastError();
     }
-    // few blocks: tiles of 32 output channels put twice as many CUs to work (each block still transforms all K inputs)
-    if (pick == 2 && logDY == 8 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
-        return launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 2 && logDY == 8) return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 2 && logDY == 7 && (algo == 4 || (algo == 0 && S * (N / 32) <= cu_count())))
-        return launch_fused_mfma<7, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 2 && logDY == 7) return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 3 && logDY == 8) return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 3 && logDY == 7) return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 3 && logDY == 9) return launch_fused_mfma<9, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 3 && logDY == 10) return launch_fused_mfma<10, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 2 && logDY == 9) return launch_fused_mfma<9, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
-    if (pick == 2 && logDY == 10) return launch_fused_mfma<10, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
-    return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream, keep_y);
+    case kFused1dMfma512Tile32:
+        return logDY == 8 ? launch_fused_mfma<8, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y)
+                          : launch_fused_mfma<7, 512, 32>(S, N, K, x, W, y, alpha, stream, keep_y);
+    case kFused1dMfma512:
+        switch (logDY) {
+        case 7: return launch_fused_mfma<7, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+        case 8: return launch_fused_mfma<8, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+        case 9: return launch_fused_mfma<9, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+        default: return launch_fused_mfma<10, 512>(S, N, K, x, W, y, alpha, stream, keep_y);
+        }
+    case kFused1dMfma256:
+        switch (logDY) {
+        case 7: return launch_fused_mfma<7, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+        case 8: return launch_fused_mfma<8, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+        case 9: return launch_fused_mfma<9, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+        default: return launch_fused_mfma<10, 256>(S, N, K, x, W, y, alpha, stream, keep_y);
+        }
+    default: return dispatch_fused_1d<true, true>(logDY, S, N, K, x, W, y, alpha, make_float2(0.f, 0.f), stream, keep_y);
+    }
 }
 
 hipError_t launch_fused_fft_cgemm(int logDY, long S, int N, int K, const float2* x, const float2* W, float2* C,

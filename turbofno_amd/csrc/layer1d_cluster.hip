@@ -16,12 +16,20 @@
 // blocks with ids less than 8 P away, all of which the in-order dispatcher has started or will start without this
 // block's resources, whatever the grid size.
 //
-// Publication protocol: partials are written with device-scope stores (written through, complete when the wave's
-// store counter drains) and read with device-scope loads (never served from a stale private line), so no cache-wide
-// write-back or invalidate is needed: the producer waits for its stores, the block's first thread bumps the
-// cluster's arrival counter, consumers poll that counter. The counter is never reset: every launch adds exactly 8
-// (8 / P per member), launches that share a counter are ordered by their stream, so an arriving member that reads the
+// Publication protocol: partials are written with relaxed device-scope atomic stores and read with relaxed device-scope
+// atomic loads; what orders them is the arrival counter of the cluster: after a block barrier the block's first thread
+// adds to it with RELEASE semantics, consumers poll it (relaxed) and then pass an ACQUIRE fence, both at device scope,
+// and a second block barrier hands the result to the other waves. The counter is never reset: every launch adds exactly
+// 8 (8 / P per member), launches that share a counter are ordered by their stream, so an arriving member that reads the
 // old value v knows the launch is complete at (v / 8 + 1) 8. That also makes the kernel replayable from a captured graph.
+//
+// Every wait is bounded. A member whose wait runs out does not use the exchange at all: it transforms the channels of
+// the other members itself and adds their products to its own output channels (a plain loop, slower, same result up to
+// summation order), so the output of a launch is valid whether or not its members ever ran side by side. It also counts
+// the event in the exchange buffer, where turbofno_exchange_status finds it.
+//
+// The exchange memory belongs to the CALLER (turbofno_exchange_attach): nothing in this file allocates, frees or
+// synchronises.
 #include "group_fft.h"
 #include "kernels.h"
 
@@ -58,7 +66,6 @@ namespace {
 constexpr int kArriveStride = 32;                               // counters 128 bytes apart: one line per cluster
 
 __device__ __forceinline__ unsigned counter_load(const unsigned* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void stores_complete() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ cpx load_published(const cpx* p)
 {
     const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -72,8 +79,8 @@ __device__ __forceinline__ void store_published(cpx* p, cpx v)
 
 }  // namespace
 
-// part[S][P][N][64]: partial products by (signal set, producing member); arrive[S * kArriveStride]; *gave_up (host
-// memory the device can write) is set when a wait ran into its bound, after which the output of that launch is invalid.
+// part[S][P][N][64]: partial products by (signal set, producing member); arrive[S * kArriveStride]; *gave_up counts the
+// members whose wait ran into its bound and which therefore computed the other members' share themselves.
 template <int NT, int KC_>
 __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S, int K, int P, const float2* __restrict__ x,
                                                                           const float2* __restrict__ W, float2* __restrict__ y,
@@ -183,39 +190,85 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
         }
         if (!last) __syncthreads();                             // sA / sW are free again for the next chunk
     }
-    stores_complete();
-    __syncthreads();
+    __shared__ unsigned s_alone;                                // set when this member's wait ran out
+    __syncthreads();                                            // every wave's partials precede the release below
     if (tid == 0) {
         unsigned* ctr = arrive + s * kArriveStride;
         // every member adds 8 / P, every launch 8 whatever its cluster size: launches with different P may follow each
         // other on a stream. 8 divides 2^32: consistent under wrap-around.
-        const unsigned old = __hip_atomic_fetch_add(ctr, 8u / (unsigned)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned add = 8u / (unsigned)P;
+        const unsigned old = __hip_atomic_fetch_add(ctr, add, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         const unsigned target = (old / 8u + 1u) * 8u;
-        if ((int)(counter_load(ctr) - target) < 0) {
-            const unsigned long long t0 = wall_clock64();
-            while ((int)(counter_load(ctr) - target) < 0) {
-                if (wall_clock64() - t0 > wait_ticks) {
-                    __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    break;
+        unsigned alone = 0;
+        if (old + add != target) {                              // not the last member to arrive
+            // a bound of zero means "do not wait": every member but the last goes on alone, whatever the timing
+            // (the host-side tests of that path rely on it)
+            if (wait_ticks == 0) alone = 1;
+            else {
+                const unsigned long long t0 = wall_clock64();
+                while ((int)(counter_load(ctr) - target) < 0) {
+                    if (wall_clock64() - t0 > wait_ticks) { alone = 1; break; }
+                    __builtin_amdgcn_s_sleep(2);
                 }
-                __builtin_amdgcn_s_sleep(2);
+            }
+            if (alone) __hip_atomic_fetch_add(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");      // pairs with the other members' release
+        s_alone = alone;
+    }
+    __syncthreads();
+    const bool alone = s_alone != 0;                            // uniform over the block
+
+    cpx c[4];
+    const int n = NB * q + (g < NB ? g : 0);
+    if (g < NB) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) c[a] = sC[g * PC + t + 16 * a];
+    }
+    if (!alone) {
+        if (g < NB) {
+            for (int qq = 1; qq < P; ++qq) {
+                const int from = (q + qq) & (P - 1);
+                const float2* p = part + ((long)(s * P + from) * N + n) * 64 + t;
+#pragma unroll
+                for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], load_published(p + 16 * a));
+            }
+        }
+    } else {
+        // The other members did not arrive in time: their share of the contraction, for this member's output channels
+        // only, from x and W. Chunks of KC channels as above (forward transforms -> sA), then lane group g adds
+        // alpha W[k][n] A[k][m] over the chunk for its channel n, in the register layout the backward pass takes.
+        for (int qq = 1; qq < P; ++qq) {
+            const int from = (q + qq) & (P - 1);
+            for (int kc = 0; kc < KB; kc += KC) {
+                const int k0 = from * KB + kc;
+                cpx out[4];
+                if (g < KC) {
+                    const float2* p = x + ((long)(k0 + g) * S + s) * DY + t;
+                    cpx vv[16], gg[16];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) vv[i] = p[16 * i];
+                    fwd_pass1(vv, tw, gg);
+                    group_forward_finish<8>(gg, exch, t, out);
+                }
+                __syncthreads();                                // all exchanges done: sA may overwrite them
+                if (g < KC) {
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) sA[g * PA + t + 16 * a] = out[a];
+                }
+                __syncthreads();
+                if (g < NB) {
+                    for (int k = 0; k < KC; ++k) {
+                        const float2 w = cmul(W[(k0 + k) + (long)n * K], alpha);
+#pragma unroll
+                        for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], cmul(sA[k * PA + t + 16 * a], w));
+                    }
+                }
+                __syncthreads();                                // sA is free again
             }
         }
     }
-    __syncthreads();
-    asm volatile("" ::: "memory");                              // the loads below are issued after the counter was seen
-
     if (g < NB) {
-        const int n = NB * q + g;
-        cpx c[4];
-#pragma unroll
-        for (int a = 0; a < 4; ++a) c[a] = sC[g * PC + t + 16 * a];
-        for (int qq = 1; qq < P; ++qq) {
-            const int from = (q + qq) & (P - 1);
-            const float2* p = part + ((long)(s * P + from) * N + n) * 64 + t;
-#pragma unroll
-            for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], load_published(p + 16 * a));
-        }
         cpx yv[16];
         group_backward<8>(c, tw, exch, t, yv);
         float2* dst = y + ((long)n * S + s) * DY + t;
@@ -225,22 +278,41 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// Exchange memory: one buffer per (device, stream) that has used this path, kept until the process ends. Calls on one stream are ordered and may share it; calls on different streams get different buffers.
+// Exchange memory: caller-owned, one buffer per (device, stream), registered with exchange_attach and forgotten with a
+// null attach. Layout of a buffer for a device of `cus` compute units (a clustered grid is at most one block per CU and
+// N at most 128, so part[S][P][N][64] never exceeds 64 KiB per CU):
+//   [0, 64 KiB * cus)                 partial products
+//   [.., + 128 B * cus)               arrival counters, one 128-byte line per cluster
+//   [.., + 256 B)                     word 0: members whose wait ran out since the last exchange_gave_up
+// Calls on one stream are ordered and share the stream's buffer; calls on different streams use different buffers.
 namespace {
 
 struct Exchange {
     float2* part = nullptr;
-    size_t part_bytes = 0;
     unsigned* arrive = nullptr;
-    long clusters = 0;
-    unsigned* gave_up = nullptr;    // pinned host word, written by a kernel whose wait ran into its bound
+    unsigned* gave_up = nullptr;
+    long clusters = 0;              // compute units the buffer was sized for
 };
 
 std::mutex g_exchange_mutex;
 // key: device, stream handle, and - for hipStreamPerThread, one handle that names a different stream in every host
 // thread - a hash of the calling thread
-std::map<std::tuple<int, hipStream_t, size_t>, Exchange> g_exchange;
+typedef std::tuple<int, hipStream_t, size_t> ExchangeKey;
+std::map<ExchangeKey, Exchange> g_exchange;
 std::atomic<unsigned long long> g_wait_ticks{ 200000000ull };    // 2 s of the 100 MHz wall clock
+
+constexpr size_t kPartBytesPerCu = sizeof(float2) * 64 * 128;
+constexpr size_t kArriveBytesPerCu = sizeof(unsigned) * kArriveStride;
+constexpr size_t kStatusBytes = 256;
+
+bool key_of(hipStream_t stream, ExchangeKey& key)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return false; }
+    const size_t thread_key = stream == hipStreamPerThread ? std::hash<std::thread::id>()(std::this_thread::get_id()) : 0;
+    key = std::make_tuple(dev, stream, thread_key);
+    return true;
+}
 
 bool stream_is_capturing(hipStream_t stream)
 {
@@ -249,51 +321,29 @@ bool stream_is_capturing(hipStream_t stream)
     return st != hipStreamCaptureStatusNone;
 }
 
-// Returns the buffer of (current device, stream); nullptr when it cannot be provided (allocation failed, or it would have
-// to be allocated while the stream is being captured). It is allocated once, at the largest size any launch can need
-// (a grid is at most one block per CU, N at most 128), and never freed or moved afterwards: a captured launch holds
-// its address.
-Exchange* exchange_for(hipStream_t stream, long clusters, size_t bytes_per_cluster)
+// stream-ordered clear (a kernel, not a memset node: this may be recorded into a graph by a capturing caller)
+__global__ void zero_words_kernel(unsigned* p, long n)
 {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// the buffer of (current device, stream), by value; false when none is attached or it is too small for `clusters`
+bool exchange_for(hipStream_t stream, long clusters, size_t bytes_per_cluster, Exchange& out)
+{
+    ExchangeKey key;
+    if (!key_of(stream, key)) return false;
     std::lock_guard<std::mutex> lock(g_exchange_mutex);
-    const size_t thread_key = stream == hipStreamPerThread ? std::hash<std::thread::id>()(std::this_thread::get_id()) : 0;
-    Exchange& e = g_exchange[std::make_tuple(dev, stream, thread_key)];
-    const size_t need = (size_t)clusters * bytes_per_cluster;
-    if (e.part && e.arrive && e.gave_up) return (e.part_bytes >= need && e.clusters >= clusters) ? &e : nullptr;
-    if (stream_is_capturing(stream)) return nullptr;
-    const long cus = cu_count();
-    const size_t part_bytes = sizeof(float2) * 64 * 128 * (size_t)cus;          // part[S][P][N][64] with S P <= cus, N <= 128
-    const size_t arrive_bytes = sizeof(unsigned) * kArriveStride * (size_t)cus;
-    if (need > part_bytes || clusters > cus) return nullptr;
-    if (!e.gave_up) {
-        if (hipHostMalloc(reinterpret_cast<void**>(&e.gave_up), 64, hipHostMallocDefault) != hipSuccess) {
-            (void)hipGetLastError();
-            e.gave_up = nullptr;
-            return nullptr;
-        }
-        *e.gave_up = 0;
-    }
-    if (!e.part) {
-        if (hipMalloc(reinterpret_cast<void**>(&e.part), part_bytes) != hipSuccess) { (void)hipGetLastError(); e.part = nullptr; return nullptr; }
-        e.part_bytes = part_bytes;
-    }
-    if (!e.arrive) {
-        if (hipMalloc(reinterpret_cast<void**>(&e.arrive), arrive_bytes) != hipSuccess) { (void)hipGetLastError(); e.arrive = nullptr; return nullptr; }
-        if (hipMemset(e.arrive, 0, arrive_bytes) != hipSuccess) {                // synchronous, once
-            (void)hipGetLastError();
-            (void)hipFree(e.arrive);
-            e.arrive = nullptr;
-            return nullptr;
-        }
-        e.clusters = cus;
-    }
-    return &e;
+    const auto it = g_exchange.find(key);
+    if (it == g_exchange.end()) return false;
+    const Exchange& e = it->second;
+    if (clusters > e.clusters || (size_t)clusters * bytes_per_cluster > kPartBytesPerCu * (size_t)e.clusters) return false;
+    out = e;
+    return true;
 }
 
 template <int NT, int KC>
-hipError_t launch_cluster_t(long S, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha, Exchange* e,
+hipError_t launch_cluster_t(long S, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha, const Exchange& e,
                             hipStream_t stream)
 {
     using G = GeoCluster<NT, KC>;
@@ -303,36 +353,91 @@ hipError_t launch_cluster_t(long S, int K, int P, const float2* x, const float2*
         return err;
     const long blocks = ((S + 7) / 8) * 8 * P;
     hipLaunchKernelGGL((fused_fft_mfma_ifft_cluster_kernel<NT, KC>), dim3((unsigned)blocks), dim3(512), G::LDS_BYTES, stream, (int)S, K, P,
-                       x, W, y, alpha, e->part, e->arrive, e->gave_up, g_wait_ticks.load(std::memory_order_relaxed));
+                       x, W, y, alpha, e.part, e.arrive, e.gave_up, g_wait_ticks.load(std::memory_order_relaxed));
     return hipGetLastError();
 }
 
 }  // namespace
 
-// Cluster size for (S, N, K), or 0 when this kernel does not apply: N in {64, 128}, every member gets a multiple of eight
-// input channels and 8 ... 32 output channels, and the whole grid is resident at once (one block per CU).
-int cluster_size_1d(int logDY, long S, int N, int K)
+size_t exchange_bytes(long cus)
+{
+    if (cus <= 0) cus = cu_count();
+    return (kPartBytesPerCu + kArriveBytesPerCu) * (size_t)cus + kStatusBytes;
+}
+
+// Registers `buffer` (exchange_bytes() bytes, 256-byte aligned, device memory of the current device) for clustered
+// launches on `stream` and clears its counters with a kernel on that stream; a null buffer forgets the stream's buffer.
+// hipErrorInvalidValue: misaligned or too small; hipErrorStreamCaptureUnsupported: the stream is being captured.
+hipError_t exchange_attach(hipStream_t stream, void* buffer, size_t bytes)
+{
+    ExchangeKey key;
+    if (!key_of(stream, key)) return hipErrorInvalidDevice;
+    if (!buffer) {
+        std::lock_guard<std::mutex> lock(g_exchange_mutex);
+        g_exchange.erase(key);
+        return hipSuccess;
+    }
+    const long cus = cu_count();
+    if (((size_t)buffer & 255) || bytes < exchange_bytes(cus)) return hipErrorInvalidValue;
+    if (stream_is_capturing(stream)) return hipErrorStreamCaptureUnsupported;
+    Exchange e;
+    e.part = static_cast<float2*>(buffer);
+    e.arrive = reinterpret_cast<unsigned*>(static_cast<char*>(buffer) + kPartBytesPerCu * (size_t)cus);
+    e.gave_up = reinterpret_cast<unsigned*>(static_cast<char*>(buffer) + (kPartBytesPerCu + kArriveBytesPerCu) * (size_t)cus);
+    e.clusters = cus;
+    const long words = (long)((kArriveBytesPerCu * (size_t)cus + kStatusBytes) / sizeof(unsigned));
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, e.arrive, words);
+    if (hipError_t err = hipGetLastError(); err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(g_exchange_mutex);
+    g_exchange[key] = e;
+    return hipSuccess;
+}
+
+bool exchange_attached(hipStream_t stream)
+{
+    ExchangeKey key;
+    if (!key_of(stream, key)) return false;
+    std::lock_guard<std::mutex> lock(g_exchange_mutex);
+    return g_exchange.find(key) != g_exchange.end();
+}
+
+// Waits for the stream, then returns (and clears) the number of cluster members whose wait has run out since the last
+// call. hipErrorNotReady: no buffer attached to the stream.
+hipError_t exchange_gave_up(hipStream_t stream, unsigned* count)
+{
+    Exchange e;
+    if (!exchange_for(stream, 0, 0, e)) return hipErrorNotReady;
+    unsigned host = 0;
+    if (hipError_t err = hipMemcpyAsync(&host, e.gave_up, sizeof(unsigned), hipMemcpyDeviceToHost, stream); err != hipSuccess) return err;
+    if (hipError_t err = hipStreamSynchronize(stream); err != hipSuccess) return err;
+    if (host) {
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, stream, e.gave_up, 1L);
+        if (hipError_t err = hipGetLastError(); err != hipSuccess) return err;
+    }
+    *count = host;
+    return hipSuccess;
+}
+
+// Cluster size for (S, N, K) on `cus` compute units, or 0 when this kernel does not apply: N in {64, 128}, every member
+// gets a multiple of eight input channels and 8 ... 32 output channels, and the whole grid is resident at once (one
+// block per CU).
+int cluster_size_1d(int logDY, long S, int N, int K, long cus)
 {
     if (logDY != 8 || (N != 64 && N != 128) || S <= 0) return 0;
-    const long cus = cu_count(), groups = (S + 7) / 8 * 8;
+    const long groups = (S + 7) / 8 * 8;
     int P = 0;
     for (int c = N / 32; c <= 8; c *= 2)                        // the largest cluster that still gives every block a CU
         if (groups * c <= cus && K % (8 * c) == 0 && N / c >= 8) P = c;
     return P;
 }
 
-// hipErrorNotReady: the exchange buffer could not be provided (the caller falls back on a kernel without one);
-// hipErrorLaunchTimeOut: an earlier launch on this stream gave up waiting for a cluster member (reported once).
+// hipErrorNotReady: no exchange buffer is attached to this stream (the caller falls back on a kernel without one)
 hipError_t launch_fused_cluster(long S, int N, int K, int P, const float2* x, const float2* W, float2* y, float2 alpha,
                                 hipStream_t stream)
 {
     if (P < 2 || P > 8 || (P & (P - 1)) || K % (8 * P) || N % P || N / P > 32 || N / P < 8) return hipErrorInvalidValue;
-    Exchange* e = exchange_for(stream, S, sizeof(float2) * 64 * (size_t)N * P);
-    if (!e) return hipErrorNotReady;
-    if (*static_cast<volatile unsigned*>(e->gave_up)) {          // reported once; the arrival counters stay consistent
-        *e->gave_up = 0;
-        return hipErrorLaunchTimeOut;
-    }
+    Exchange e;
+    if (!exchange_for(stream, S, sizeof(float2) * 64 * (size_t)N * P, e)) return hipErrorNotReady;
     // chunk = the largest of 32 / 16 / 8 channels that divides a member's share
     const int KB = K / P, KC = KB % 32 == 0 ? 32 : (KB % 16 == 0 ? 16 : 8);
     if (N == 128 && KC == 32) return launch_cluster_t<128, 32>(S, K, P, x, W, y, alpha, e, stream);

@@ -36,11 +36,32 @@
 
 struct Problem { int bs, dx, dy, n, k; };
 
+// a positional argument as a positive integer; anything else (text, trailing characters, zero, overflow) ends the run
+static int positive_int(const char* text, const char* name)
+{
+    char* end = nullptr;
+    const long v = strtol(text, &end, 10);
+    if (end == text || *end != '\0' || v <= 0 || v > 0x7fffffffL) {
+        fprintf(stderr, "argument %s = \"%s\" is not a positive integer\n", name, text);
+        exit(EXIT_FAILURE);
+    }
+    return (int)v;
+}
+
+// log2 of a transform length the kernels are built for (128 ... 1024), or -1
+static int log2_of_length(int v)
+{
+    for (int l = 7; l <= 10; ++l)
+        if (v == (1 << l)) return l;
+    return -1;
+}
+
 static std::vector<Problem> problems_from(int argc, char** argv)
 {
     std::vector<Problem> out;
     if (argc == 6) {
-        out.push_back({ atoi(argv[1]), atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]) });
+        out.push_back({ positive_int(argv[1], "bs"), positive_int(argv[2], TURBOFNO_VARIANT_2D ? "DX" : "dimX"),
+                        positive_int(argv[3], "DY"), positive_int(argv[4], "N"), positive_int(argv[5], "K") });
         return out;
     }
     auto cfg = load_problem_config(argc == 2 ? argv[1] : DEFAULT_CONFIG_PATH);
@@ -65,8 +86,33 @@ int main(int argc, char** argv)
     // measurement aid of these executables only (the library itself reads no environment): forces one of the fused 1D kernels
     if (const char* e = getenv("TURBOFNO_1D_ALGO")) CHECK_TURBOFNO(turbofno_set_1d_algo(atoi(e)));
 
-    for (const Problem& p : problems_from(argc, argv)) {
+    const std::vector<Problem> problems = problems_from(argc, argv);     // argument errors end the run before any HIP call
+
+    // Like every other buffer of the run, the exchange memory of the clustered 1D kernel (small grids with 64 channels or
+    // more) belongs to this main: allocated once, attached to the default stream, which all launches below use.
+    // TURBOFNO_NO_EXCHANGE=1 leaves it out (the library then runs kernels that need none).
+    void* exchange = nullptr;
+    if (TURBOFNO_VARIANT == 'D' && !getenv("TURBOFNO_NO_EXCHANGE")) {
+        const size_t bytes = turbofno_exchange_bytes(0);
+        HIP_RT_CALL(hipMalloc(&exchange, bytes));
+        if (exchange) CHECK_TURBOFNO(turbofno_exchange_attach(nullptr, exchange, bytes));
+    }
+
+    for (const Problem& p : problems) {
         if (p.k % THREADBLOCK_K != 0) { fprintf(stderr, "K=%d is not a multiple of %d: problem skipped\n", p.k, THREADBLOCK_K); continue; }
+        if (p.bs <= 0 || p.dx <= 0 || p.n <= 0 || p.k <= 0 || p.n % THREADBLOCK_M != 0) {
+            fprintf(stderr, "bs=%d, %s=%d, N=%d, K=%d: sizes must be positive and N a multiple of %d: problem skipped\n", p.bs,
+                    TURBOFNO_VARIANT_2D ? "DX" : "dimX", p.dx, p.n, p.k, THREADBLOCK_M);
+            continue;
+        }
+        // transform lengths index the kernel tables by log2(length) - 7: only exact powers of two from 128 to 1024 have an
+        // entry (a rounded logarithm would run a kernel of another length on these buffers)
+        const int logDY = log2_of_length(p.dy), logDX = TURBOFNO_VARIANT_2D ? log2_of_length(p.dx) : 0;
+        if (logDY < 0 || logDX < 0) {
+            fprintf(stderr, "DY=%d%s: transform lengths must be 128, 256, 512 or 1024: problem skipped\n", p.dy,
+                    TURBOFNO_VARIANT_2D ? (", DX=" + std::to_string(p.dx)).c_str() : "");
+            continue;
+        }
         // 1D: x[K][bs*dimX][DY]; 2D: x[K][bs][DX][DY]
         const size_t per_channel = TURBOFNO_VARIANT_2D ? (size_t)p.bs * p.dx * p.dy : (size_t)p.bs * p.dx * p.dy;
         const size_t in_elems = per_channel * p.k, out_elems = per_channel * p.n, w_elems = (size_t)p.k * p.n;
@@ -93,7 +139,6 @@ int main(int argc, char** argv)
         // intermediates t1[K*bs][64][DY], t2[N*bs][64][DY]
         const long S = TURBOFNO_VARIANT_2D ? (long)p.bs * THREADBLOCK_M : (long)p.bs * p.dx;   // signals per channel of the Y stage
         const long M = THREADBLOCK_M * S;
-        const int logDY = (int)lround(log2((double)p.dy)), logDX = (int)lround(log2((double)p.dx));
         void *dA = nullptr, *dC = nullptr, *t1 = nullptr, *t2 = nullptr;
         if (TURBOFNO_VARIANT != 'D') {
             HIP_RT_CALL(hipMalloc(&dA, sizeof(float) * 2 * M * p.k));
@@ -167,6 +212,14 @@ int main(int argc, char** argv)
         if (dC) HIP_RT_CALL(hipFree(dC));
         if (t1) HIP_RT_CALL(hipFree(t1));
         if (t2) HIP_RT_CALL(hipFree(t2));
+    }
+    if (exchange) {
+        unsigned gave_up = 0;
+        if (turbofno_exchange_status(nullptr, &gave_up) == TURBOFNO_ERR_EXCHANGE)
+            fprintf(stderr, "note: %u cluster member(s) ran out of their wait during this run (results valid, those launches slow)\n", gave_up);
+        CHECK_TURBOFNO(turbofno_exchange_detach(nullptr));
+        HIP_RT_CALL(hipDeviceSynchronize());
+        HIP_RT_CALL(hipFree(exchange));
     }
     return 0;
 }
