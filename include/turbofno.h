@@ -176,8 +176,8 @@ int turbofno_get_1d_algo(void);
  *                                 device): 64 KiB + 128 B per compute unit + 256 B (16.03 MiB on 256 CUs);
  *   turbofno_exchange_attach      registers `buffer` (device memory, 256-byte aligned, at least that size) for the 1D
  *                                 layer calls on `stream` of the current device and clears its counters with a small
- *                                 kernel on that stream (no allocation, no synchronisation). Not inside a capture of
- *                                 that stream. Attaching again replaces the buffer;
+ *                                 kernel on that stream (no allocation, no synchronisation). Not inside a capture of that
+ *                                 stream. Attaching again replaces the buffer;
  *   turbofno_exchange_detach      forgets it. Detach before freeing the buffer or destroying the stream; work already
  *                                 enqueued (or captured into a graph) keeps using the memory until it has run.
  * While a buffer is attached, turbofno_fused_fft_cgemm_ifft / turbofno_layer_1d on that stream (and the middle stage of
@@ -185,15 +185,17 @@ int turbofno_get_1d_algo(void);
  * no exchange. Calls on one stream are ordered and share its buffer; use one buffer per stream, never one buffer on two
  * streams. A graph captured on the stream holds the buffer's address: do not replay it concurrently with other 1D
  * layer calls that use the same buffer.
- * Results do not depend on the exchange working: every inter-block wait is bounded (default 2 s,
- * turbofno_set_exchange_wait_us, process-wide; 0 = do not wait at all, for tests), and a cluster member whose wait runs
- * out computes the other members' share itself, so the output of every launch is valid - only late. Such events are
- * counted in the buffer:
- *   turbofno_exchange_status      WAITS for the work enqueued on `stream`, then stores the number of members that ran
- *                                 out of their wait since the last call in *gave_up (may be NULL) and clears it;
- *                                 returns TURBOFNO_ERR_EXCHANGE when that number is not zero (advisory: the clustered
- *                                 kernel does not suit the way this process shares the GPU), TURBOFNO_OK otherwise and
- *                                 when no buffer is attached.
+ * Results do not depend on the exchange working: every inter-block wait is bounded (default 100 us,
+ * turbofno_set_exchange_wait_us, process-wide; 0 = never wait: every member works alone, for tests), and a cluster
+ * member that does not get the other members' partial products in time - or that starts so late that the others are
+ * already publishing theirs, as can happen on the first launch after the GPU has been idle - computes their share
+ * itself, so the output of every launch is valid, only later (by some 15 - 50 us, plus the wait if it came to that).
+ * Such a member counts itself in the buffer:
+ *   turbofno_exchange_status      WAITS for the work enqueued on `stream`, stores the count since the last call in
+ *                                 *gave_up (may be NULL) and clears it; returns TURBOFNO_ERR_EXCHANGE when the count
+ *                                 was not zero (advisory: the members of a cluster did not run side by side, i.e. the
+ *                                 clustered kernel does not suit the way this process shares the GPU; detach the
+ *                                 buffer to stop using it), TURBOFNO_OK otherwise and when no buffer is attached.
  */
 size_t turbofno_exchange_bytes(int compute_units);
 int turbofno_exchange_attach(void* stream, void* buffer, size_t bytes);

@@ -105,7 +105,7 @@ int turbofno_get_1d_algo(void) { return algo_1d(); }
 
 int turbofno_set_exchange_wait_us(unsigned long long microseconds)
 {
-    tfno::set_cluster_wait_ticks(microseconds > (~0ull) / 100 ? ~0ull : microseconds * 100);   // 100 MHz wall clock
+    tfno::set_cluster_wait_ticks(microseconds > (~0ull) / 100 ? ~0ull : microseconds * 100);   // 100 MHz wall clock   // 100 MHz wall clock
     return TURBOFNO_OK;
 }
 
@@ -136,8 +136,9 @@ int turbofno_exchange_status(void* stream, unsigned* gave_up)
     if (int rc = hip_status(e, "exchange_status")) return rc;
     if (gave_up) *gave_up = count;
     if (count)
-        return fail(TURBOFNO_ERR_EXCHANGE, "%u cluster member(s) on this stream ran out of their wait and computed the other members' share "
-                                           "themselves (results are valid; the launches were slow)", count);
+        return fail(TURBOFNO_ERR_EXCHANGE, "%u cluster member(s) on this stream did not get the other members' partial products in time "
+                                           "and computed their share themselves since the last call: results are valid, those "
+                                           "launches were slow", count);
     return TURBOFNO_OK;
 }
 

@@ -16,20 +16,39 @@
 // blocks with ids less than 8 P away, all of which the in-order dispatcher has started or will start without this
 // block's resources, whatever the grid size.
 //
-// Publication protocol: partials are written with relaxed device-scope atomic stores and read with relaxed device-scope
-// atomic loads; what orders them is the arrival counter of the cluster: after a block barrier the block's first thread
-// adds to it with RELEASE semantics, consumers poll it (relaxed) and then pass an ACQUIRE fence, both at device scope,
-// and a second block barrier hands the result to the other waves. The counter is never reset: every launch adds exactly
-// 8 (8 / P per member), launches that share a counter are ordered by their stream, so an arriving member that reads the
-// old value v knows the launch is complete at (v / 8 + 1) 8. That also makes the kernel replayable from a captured graph.
+// Publication protocol: every partial product is one 64-bit word that says by itself whether it has been written in
+// THIS launch. At the start of the kernel, long before anything is published, each consumer lane overwrites the words it
+// will read at the end with a sentinel (all bits set: a NaN pattern that arithmetic on finite data never produces);
+// producers later overwrite them with their partial products; the consumer reads each word until it no longer holds the
+// sentinel. All of these are relaxed device-scope atomic accesses to one location each, and the argument needs nothing
+// more than the coherence of a single location: the consumer's read comes after its own sentinel store in program order,
+// so it returns that sentinel or a value stored later in the word's modification order - which can only be this
+// launch's product (launches on a stream are ordered, a word has one producer per launch); whatever an earlier launch,
+// of whatever shape, left in the buffer is wiped before it can be read. If a product lands BEFORE the sentinel (a
+// consumer that started seconds after its producers), the consumer never sees it and falls back as described below:
+// slow, never wrong. No ordering between different locations is needed, hence no release / acquire fences (at device
+// scope those write back and invalidate the whole L2 of the XCD: +2.6 us on a 16 us kernel, measured), no counter that
+// correctness depends on, and the kernel is replayable from a captured graph.
+// Two counters per cluster are timing hints and nothing else. The ANNOUNCE counter guards the one weak spot of the
+// scheme, a consumer that starts after its producers have published (a grid that is not resident all at once): each
+// member adds to it just before it publishes its first word, and a consumer wavefront that finds it off a multiple of 8
+// at its start knows that a member of this launch is already publishing; it then neither wipes nor reads but leaves its
+// channels to the fallback at once instead of waiting out the bound for words it may have wiped. The ARRIVAL counter
+// tells the members WHEN to read: words requested while their
+// producer's stores are still on their way miss the L2 and take 3 us instead of 0.6 to come back, so each member adds
+// to the counter when its own stores have completed and reads once all have done so (or 20 us have passed). The counter
+// is never reset: every launch adds exactly 8 to each counter (8 / P per member), launches are ordered by their stream,
+// so a member that reads the old value v knows all have arrived at (v / 8 + 1) 8. All counter accesses are relaxed; a
+// counter that is early, late or out of step only costs time.
 //
-// Every wait is bounded. A member whose wait runs out does not use the exchange at all: it transforms the channels of
-// the other members itself and adds their products to its own output channels (a plain loop, slower, same result up to
-// summation order), so the output of a launch is valid whether or not its members ever ran side by side. It also counts
-// the event in the exchange buffer, where turbofno_exchange_status finds it.
+// Every wait is bounded. A wavefront that does not get all its words in time leaves them; when the block has stored
+// what it could, it transforms the channels of the other members itself and adds their products to its own output
+// channels (a plain loop, slower, same result up to summation order) and stores y again, so the output of a launch is
+// valid whether or not its members ever ran side by side. Each such member counts itself in the exchange buffer, where
+// turbofno_exchange_status finds the number.
 //
 // The exchange memory belongs to the CALLER (turbofno_exchange_attach): nothing in this file allocates, frees or
-// synchronises.
+// synchronises, except that reading the status waits for the stream.
 #include "group_fft.h"
 #include "kernels.h"
 
@@ -64,23 +83,74 @@ template <int NT, int KC_> struct GeoCluster {
 namespace {
 
 constexpr int kArriveStride = 32;                               // counters 128 bytes apart: one line per cluster
+constexpr unsigned long long kHintTicks = 2000;                 // 20 us of the 100 MHz clock: longest wait for the arrival hint
+constexpr unsigned long long kUnwritten = ~0ull;               // the sentinel: both halves a NaN with all payload bits set
 
-__device__ __forceinline__ unsigned counter_load(const unsigned* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ cpx load_published(const cpx* p)
+__device__ __forceinline__ unsigned long long load_published(const cpx* p)
 {
-    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return __builtin_bit_cast(cpx, v);
+    return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void store_published(cpx* p, cpx v)
+__device__ __forceinline__ void store_published(cpx* p, unsigned long long v)
 {
-    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace
 
-// part[S][P][N][64]: partial products by (signal set, producing member); arrive[S * kArriveStride]; *gave_up counts the
-// members whose wait ran into its bound and which therefore computed the other members' share themselves.
+// The 4 (P - 1) words a lane reads from the other members (its channel's modes t + 16 a in each member's part).
+// wipe_inbox: the sentinel over them, at the start of the kernel.
+template <int P_> __device__ __forceinline__ void wipe_inbox(float2* base, long member_stride, int q)
+{
+#pragma unroll
+    for (int qq = 1; qq < P_; ++qq) {
+        float2* p = base + (long)((q + qq) & (P_ - 1)) * member_stride;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) store_published(p + 16 * a, kUnwritten);
+    }
+}
+// take_partials: all of them requested at once; words that still hold the sentinel are requested again until `wait_ticks`
+// of the 100 MHz clock have passed. On success they are added to c. The decision is per wavefront.
+template <int P_>
+__device__ __forceinline__ bool take_partials(float2* base, long member_stride, int q, cpx (&c)[4], unsigned long long wait_ticks)
+{
+    unsigned long long f[P_ - 1][4];
+#pragma unroll
+    for (int qq = 1; qq < P_; ++qq) {
+        float2* p = base + (long)((q + qq) & (P_ - 1)) * member_stride;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) f[qq - 1][a] = load_published(p + 16 * a);
+    }
+    auto missing = [&]() {
+        bool m = false;
+#pragma unroll
+        for (int qq = 0; qq < P_ - 1; ++qq)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) m |= f[qq][a] == kUnwritten;
+        return m;
+    };
+    if (__any(missing())) {
+        const unsigned long long t0 = wall_clock64();
+        do {
+            if (wall_clock64() - t0 > wait_ticks) return false;
+            __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+            for (int qq = 1; qq < P_; ++qq) {
+                float2* p = base + (long)((q + qq) & (P_ - 1)) * member_stride;
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    if (f[qq - 1][a] == kUnwritten) f[qq - 1][a] = load_published(p + 16 * a);
+            }
+        } while (__any(missing()));
+    }
+#pragma unroll
+    for (int qq = 0; qq < P_ - 1; ++qq)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], __builtin_bit_cast(cpx, f[qq][a]));
+    return true;
+}
+
+// part[S][P][N][64]: partial products by (signal set, producing member), 64-bit words; arrive[S * kArriveStride]: arrival
+// counters (a timing hint); *gave_up counts the members that computed the other members' share themselves.
 template <int NT, int KC_>
 __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S, int K, int P, const float2* __restrict__ x,
                                                                           const float2* __restrict__ W, float2* __restrict__ y,
@@ -93,6 +163,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
     float2* sA = lds;
     float* sW = reinterpret_cast<float*>(lds + G::REGION0);
     float2* sC = lds + G::REGION0 + G::REGION1;
+    __shared__ unsigned s_late;                                 // a wavefront of this block did not get its words in time
 
     const int tid = threadIdx.x;
     const int g = tid >> 4, t = tid & 15;                       // transform role: lane group g, lane t
@@ -125,19 +196,44 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
     cpx v[16];
     if (g < KC) issue(v, 0);
     float2* mine = part + ((long)(s * P + q) * N) * 64 + mt * 16 + col;
-
-    for (int kc = 0; kc < KB; kc += KC) {
-        const bool last = kc + KC >= KB;
-        // W chunk: lanes run along k, the contiguous direction of W[k + n*K]; the two halves of a wavefront take
-        // channels eight apart (eight banks apart in the tile)
-        constexpr int WPT = KC * NT / 512;                      // KB is a multiple of KC: every chunk is full
-        float2 wv[WPT];
+    // consumer role: lane group g < NB finishes output channel n; its words in the other members' parts
+    const int n = NB * q + (g < NB ? g : 0);
+    float2* inbox = part + ((long)s * P * N + n) * 64 + t;
+    const long member_stride = (long)N * 64;
+    if (tid == 0) s_late = 0;
+    // W chunk: lanes run along k, the contiguous direction of W[k + n*K]; the two halves of a wavefront take channels
+    // eight apart (eight banks apart in the tile)
+    constexpr int WPT = KC * NT / 512;                          // KB is a multiple of KC: every chunk is full
+    float2 wv[WPT];
+    auto load_w = [&](int kc) {
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * 512;
-            const int k = idx % KC, r = idx / KC, n = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
-            wv[u] = W[(kbase + kc + k) + (long)n * K];
+            const int k = idx % KC, r = idx / KC, nn = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
+            wv[u] = W[(kbase + kc + k) + (long)nn * K];
         }
+    };
+    load_w(0);
+    // The sentinel over the words this lane group will read at the end: behind the first loads of x and W (memory
+    // results come back in the order of the requests, so no load queues up behind these stores), microseconds before
+    // any member publishes - unless this block has started that late: then a member has announced itself already (the
+    // counter is off a multiple of 8), and the wavefront leaves its words alone and its channels to the fallback.
+    // The stores cost the kernel 0.9 us wherever they are placed (12 - 28 written-through stores per lane in the same
+    // queue as the partial products); this is the place with the widest margin.
+    unsigned* announce = arrive + s * kArriveStride + 1;
+    bool on_time = true;                                        // uniform over the wavefront
+    if (g < NB) {
+        const unsigned seen = __hip_atomic_load(announce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        on_time = (__builtin_amdgcn_readfirstlane(seen) & 7u) == 0u;
+        if (on_time) {
+            if (P == 2) wipe_inbox<2>(inbox, member_stride, q);
+            else if (P == 4) wipe_inbox<4>(inbox, member_stride, q);
+            else wipe_inbox<8>(inbox, member_stride, q);
+        }
+    }
+
+    for (int kc = 0; kc < KB; kc += KC) {
+        const bool last = kc + KC >= KB;
         cpx out[4];
         if (g < KC) {
             cpx gg[16];
@@ -149,19 +245,21 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * 512;
-            const int k = idx % KC, r = idx / KC, n = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
+            const int k = idx % KC, r = idx / KC, nn = (r & ~9) | ((r & 1) << 3) | ((r >> 3) & 1);
             const float c = wv[u].x * alpha.x - wv[u].y * alpha.y, d = wv[u].x * alpha.y + wv[u].y * alpha.x;
-            float* dstw = &sW[(k >> 2) * G::WGROUP + (k & 3) * G::WROW + n];
+            float* dstw = &sW[(k >> 2) * G::WGROUP + (k & 3) * G::WROW + nn];
             dstw[0] = c;
             dstw[G::WPLANE] = d - c;
             dstw[2 * G::WPLANE] = c + d;
         }
+        if (!last) load_w(kc + KC);
         __syncthreads();                                        // all exchanges done: sA may overwrite them
         if (g < KC) {
 #pragma unroll
             for (int a = 0; a < 4; ++a) sA[g * PA + t + 16 * a] = out[a];
         }
         __syncthreads();
+        if (last && tid == 0) __hip_atomic_fetch_add(announce, 8u / (unsigned)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const float2* arow = sA + kq * PA + mt * 16 + col;
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
@@ -176,68 +274,71 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
                 p3[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[2 * G::WPLANE], b.y, p3[i], 0, 0, 0);
             }
             if (last) {
-                // D[row = 4 kq + v][col]: output channel n = 16 tile + 4 kq + v, mode 16 mt + col. NB is a multiple of
-                // 8, so the four channels of a lane have one owner.
-                const int n = 16 * tile + 4 * kq;
-                const bool own = n / NB == q;
+                // D[row = 4 kq + v][col]: output channel 16 tile + 4 kq + v, mode 16 mt + col. NB is a multiple of 8, so
+                // the four channels of a lane have one owner.
+                const int nd = 16 * tile + 4 * kq;
+                const bool own = nd / NB == q;
 #pragma unroll
                 for (int vv = 0; vv < 4; ++vv) {
                     const float2 c = make_float2(p1[i][vv] - p3[i][vv], p1[i][vv] + p2[i][vv]);
-                    if (own) sC[(n + vv - NB * q) * PC + mt * 16 + col] = c;
-                    else store_published(mine + (long)(n + vv) * 64, c);
+                    if (own) sC[(nd + vv - NB * q) * PC + mt * 16 + col] = c;
+                    else store_published(mine + (long)(nd + vv) * 64, __builtin_bit_cast(unsigned long long, c));
                 }
             }
         }
         if (!last) __syncthreads();                             // sA / sW are free again for the next chunk
     }
-    __shared__ unsigned s_alone;                                // set when this member's wait ran out
-    __syncthreads();                                            // every wave's partials precede the release below
+    __syncthreads();                                            // the own product is complete in sC; own stores have completed
+    // Arrival hint (see the head of this file): every member adds 8 / P, every launch 8 whatever its cluster size, so
+    // launches with different P may follow each other on a stream; 8 divides 2^32: consistent under wrap-around.
+    // A wait bound of zero means "never wait": every member then works alone, whatever the timing (the tests of that
+    // path rely on it).
     if (tid == 0) {
         unsigned* ctr = arrive + s * kArriveStride;
-        // every member adds 8 / P, every launch 8 whatever its cluster size: launches with different P may follow each
-        // other on a stream. 8 divides 2^32: consistent under wrap-around.
         const unsigned add = 8u / (unsigned)P;
-        const unsigned old = __hip_atomic_fetch_add(ctr, add, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned old = __hip_atomic_fetch_add(ctr, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const unsigned target = (old / 8u + 1u) * 8u;
-        unsigned alone = 0;
-        if (old + add != target) {                              // not the last member to arrive
-            // a bound of zero means "do not wait": every member but the last goes on alone, whatever the timing
-            // (the host-side tests of that path rely on it)
-            if (wait_ticks == 0) alone = 1;
-            else {
-                const unsigned long long t0 = wall_clock64();
-                while ((int)(counter_load(ctr) - target) < 0) {
-                    if (wall_clock64() - t0 > wait_ticks) { alone = 1; break; }
-                    __builtin_amdgcn_s_sleep(2);
-                }
-            }
-            if (alone) __hip_atomic_fetch_add(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + add != target && wait_ticks != 0) {
+            const unsigned long long t0 = wall_clock64();
+            const unsigned long long bound = wait_ticks < kHintTicks ? wait_ticks : kHintTicks;
+            while ((int)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0 && wall_clock64() - t0 <= bound)
+                __builtin_amdgcn_s_sleep(2);
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");      // pairs with the other members' release
-        s_alone = alone;
     }
     __syncthreads();
-    const bool alone = s_alone != 0;                            // uniform over the block
 
     cpx c[4];
-    const int n = NB * q + (g < NB ? g : 0);
-    if (g < NB) {
+    auto own_product = [&]() {
 #pragma unroll
         for (int a = 0; a < 4; ++a) c[a] = sC[g * PC + t + 16 * a];
-    }
-    if (!alone) {
-        if (g < NB) {
-            for (int qq = 1; qq < P; ++qq) {
-                const int from = (q + qq) & (P - 1);
-                const float2* p = part + ((long)(s * P + from) * N + n) * 64 + t;
+    };
+    auto finish_channel = [&]() {                               // backward transform of channel n from c, y stored
+        cpx yv[16];
+        group_backward<8>(c, tw, exch, t, yv);
+        float2* dst = y + ((long)n * S + s) * DY + t;
 #pragma unroll
-                for (int a = 0; a < 4; ++a) c[a] = cadd(c[a], load_published(p + 16 * a));
-            }
+        for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, yv[i]);
+    };
+    if (g < NB) {                                               // whole wavefronts: NB is a multiple of 8 lane groups
+        bool ok = false;
+        if (wait_ticks != 0 && on_time) {
+            own_product();
+            if (P == 2) ok = take_partials<2>(inbox, member_stride, q, c, wait_ticks);
+            else if (P == 4) ok = take_partials<4>(inbox, member_stride, q, c, wait_ticks);
+            else ok = take_partials<8>(inbox, member_stride, q, c, wait_ticks);
         }
-    } else {
-        // The other members did not arrive in time: their share of the contraction, for this member's output channels
-        // only, from x and W. Chunks of KC channels as above (forward transforms -> sA), then lane group g adds
-        // alpha W[k][n] A[k][m] over the chunk for its channel n, in the register layout the backward pass takes.
+        if (ok) finish_channel();
+        else s_late = 1;
+    }
+    // Only when a wavefront was left without its words: the whole block computes the other members' share of the
+    // contraction, for this member's output channels, from x and W. Chunks of KC channels as above (forward transforms
+    // -> sA), then lane group g adds alpha W[k][n] A[k][m] over the chunk for its channel n, in the register layout the
+    // backward pass takes. Every channel of the member is stored again (those that were complete get the same values up
+    // to summation order).
+    __syncthreads();
+    if (s_late != 0) {                                          // uniform over the block
+        if (tid == 0) __hip_atomic_fetch_add(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (g < NB) own_product();
         for (int qq = 1; qq < P; ++qq) {
             const int from = (q + qq) & (P - 1);
             for (int kc = 0; kc < KB; kc += KC) {
@@ -267,13 +368,7 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
                 __syncthreads();                                // sA is free again
             }
         }
-    }
-    if (g < NB) {
-        cpx yv[16];
-        group_backward<8>(c, tw, exch, t, yv);
-        float2* dst = y + ((long)n * S + s) * DY + t;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) store_streaming(dst + 16 * i, yv[i]);
+        if (g < NB) finish_channel();
     }
 }
 
@@ -281,9 +376,9 @@ __global__ __launch_bounds__(512) void fused_fft_mfma_ifft_cluster_kernel(int S,
 // Exchange memory: caller-owned, one buffer per (device, stream), registered with exchange_attach and forgotten with a
 // null attach. Layout of a buffer for a device of `cus` compute units (a clustered grid is at most one block per CU and
 // N at most 128, so part[S][P][N][64] never exceeds 64 KiB per CU):
-//   [0, 64 KiB * cus)                 partial products
+//   [0, 64 KiB * cus)                 partial products (no initial state needed: every launch wipes what it will read)
 //   [.., + 128 B * cus)               arrival counters, one 128-byte line per cluster
-//   [.., + 256 B)                     word 0: members whose wait ran out since the last exchange_gave_up
+//   [.., + 256 B)                     word 0: members that computed the others' share themselves since the last report
 // Calls on one stream are ordered and share the stream's buffer; calls on different streams use different buffers.
 namespace {
 
@@ -299,7 +394,9 @@ std::mutex g_exchange_mutex;
 // thread - a hash of the calling thread
 typedef std::tuple<int, hipStream_t, size_t> ExchangeKey;
 std::map<ExchangeKey, Exchange> g_exchange;
-std::atomic<unsigned long long> g_wait_ticks{ 200000000ull };    // 2 s of the 100 MHz wall clock
+// Default bound of a wait: 100 us of the 100 MHz wall clock, about twice what the fallback costs - waiting longer for
+// members that are not running is slower than doing their work
+std::atomic<unsigned long long> g_wait_ticks{ 10000ull };
 
 constexpr size_t kPartBytesPerCu = sizeof(float2) * 64 * 128;
 constexpr size_t kArriveBytesPerCu = sizeof(unsigned) * kArriveStride;
@@ -321,7 +418,7 @@ bool stream_is_capturing(hipStream_t stream)
     return st != hipStreamCaptureStatusNone;
 }
 
-// stream-ordered clear (a kernel, not a memset node: this may be recorded into a graph by a capturing caller)
+// stream-ordered clear (a kernel, not a memset node)
 __global__ void zero_words_kernel(unsigned* p, long n)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -401,8 +498,8 @@ bool exchange_attached(hipStream_t stream)
     return g_exchange.find(key) != g_exchange.end();
 }
 
-// Waits for the stream, then returns (and clears) the number of cluster members whose wait has run out since the last
-// call. hipErrorNotReady: no buffer attached to the stream.
+// Waits for the stream, then returns (and clears) the number of cluster members that have computed the other members'
+// share themselves since the last call. hipErrorNotReady: no buffer attached to the stream.
 hipError_t exchange_gave_up(hipStream_t stream, unsigned* count)
 {
     Exchange e;
