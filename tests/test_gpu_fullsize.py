@@ -117,6 +117,22 @@ def test_config4_bs16_against_oracle_slices(D, K, tol):
         _check_batch_slices(y, x_h, W_h, 1 - 1j, (0, 5, 15), tol, "config4 D=%d K=%d algo %d" % (D, K, algo))
 
 
+@pytest.mark.parametrize("bs", [1, 4])
+@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("K", [16, 32])
+def test_config4_small_batches_against_oracle(bs, D, K, tol):
+    """configuration 4 at bs = 1 and 4: the algorithm chosen by size (three kernels) and the other two, every batch
+    element against the oracle; the choice itself is asserted, so that a change of the rule shows up here"""
+    assert tf.query_2d_algo(bs, D, D, K, 64) == tf.ALGO_THREE_KERNEL
+    x_h, W_h = workloads.uniform_2d(470 + bs + D + K, bs, D, D, K, 64)
+    x, W = torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
+    for algo in (0, 2, 3):
+        print("config4 small batch vs oracle", bs, D, K, "algo", algo, flush=True)
+        y = tf.layer_2d(x, W, alpha=0.5 + 1j, algo=algo)
+        torch.cuda.synchronize()
+        _check_batch_slices(y, x_h, W_h, 0.5 + 1j, range(bs), tol, "config4 bs=%d D=%d K=%d algo %d" % (bs, D, K, algo))
+
+
 @pytest.mark.parametrize("bs,DX,DY,K,N,algo", [
     (4, 512, 512, 32, 64, 0),        # whole rows first by size: 2048 row blocks of 32 rows on at most 768 persistent blocks
     (4, 256, 1024, 32, 64, 0),       # DY > DX: whole rows first, eight batches of rows per block

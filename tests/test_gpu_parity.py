@@ -272,6 +272,32 @@ def test_image_stage_entry_points(DX, DY, tol):
     check(y, np.fft.ifft2(padded, axes=(1, 2)) * (DX * DY), tol, "ifft2d_pad")
 
 
+# (S, DY, K, N, kernel the size rule picks on 256 CUs without an exchange buffer): one shape per branch of the rule
+SIZE_RULE_SHAPES = [
+    (1, 128, 8, 64, 4), (40, 256, 24, 128, 4),        # at most one 32-channel tile per CU: 512 threads, tiles of 32
+    (200, 128, 16, 64, 2), (200, 256, 40, 64, 2),     # up to one 64-channel item per CU: 512 threads
+    (300, 256, 32, 64, 3), (700, 256, 8, 64, 3),      # several items per CU: 256 threads
+    (300, 128, 32, 64, 8), (800, 128, 64, 128, 8),    # DY = 128: wide tiles
+    (1000, 256, 16, 128, 8), (300, 256, 128, 64, 8),   # DY = 256: tiles of 128 channels / 128 input channels
+    (1100, 128, 24, 64, 5), (600, 128, 8, 64, 5),     # DY = 128, several items per SIMD: one wavefront per item
+    (64, 256, 64, 128, 6), (100, 256, 96, 64, 6),     # small grids, 64 channels or more: K split over the waves of a block
+    (100, 512, 16, 64, 2), (300, 512, 16, 64, 1), (300, 1024, 64, 64, 3),   # the long lengths
+]
+
+
+@pytest.mark.parametrize("S,DY,K,N,kernel", SIZE_RULE_SHAPES)
+def test_layer_1d_size_rule_against_oracle(S, DY, K, N, kernel, tol):
+    """the kernel chosen by size, asserted through the query and checked against the oracle: one shape for every branch of
+    the rule (the clustered kernel, which needs an exchange buffer, has its own tests)"""
+    print("case size rule vs oracle", S, DY, K, N, "kernel", kernel, flush=True)
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert tf.query_1d_kernel(DY, S, N, K, compute_units=0) == kernel
+    x, W = workloads.uniform_1d(7000 + S + DY + K + N, S, DY, K, N)
+    y = tf.layer_1d(dev(x), dev(W), alpha=0.5 - 0.75j)
+    torch.cuda.synchronize()
+    check(y, oracle.layer_1d(x, W, 0.5 - 0.75j), tol, "size rule S=%d DY=%d K=%d N=%d" % (S, DY, K, N))
+
+
 def test_layer_1d_across_the_size_rule():
     """60 seeded shapes from one signal set to a few items per CU (S up to 700, all four lengths, K up to 136, N up to
     256), kernel chosen by size: crosses every branch of the choice (clustered, 512- and 256-thread blocks, one

@@ -61,8 +61,12 @@ __device__ __forceinline__ void decode_block_1d(long S, int ntiles, int DY, bool
 #endif
 
 // Share of the work of a pair of persistent blocks (2p on an even XCD, 2p + 1 on an odd one) that the even block takes in
-// the store-bound backward kernels: the odd XCDs of this GPU sustain about a fifth less store traffic than the even ones.
-constexpr int kEvenShareNum = 17, kEvenShareDen = 32;
+// the store-bound backward kernels, in parts of kEvenShareDen: 17 on MI355X (gfx950, 8 XCDs of 32 CUs), whose odd XCDs
+// sustain about a fifth less store traffic than the even ones (measured; 17 and 18 level, 19 worse); an even 16 on any
+// other part or partition, where neither that ratio nor "block parity = XCD parity" is known to hold. A kernel argument,
+// resolved per device by even_share_parts().
+constexpr int kEvenShareDen = 32;
+int even_share_parts();
 
 // compute units of the current device (cached per device)
 int cu_count();

@@ -17,6 +17,7 @@
 // lanes coincide, every access is contiguous per wavefront) and the GEMM is oblivious to it.
 #include "group_fft.h"
 #include "kernels.h"
+#include <string>
 #include <type_traits>
 
 namespace tfno {
@@ -186,14 +187,14 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
 // every launch on every box measured; a store-only probe gives the same picture), so with the same number of images per
 // block the even half of the chip idles for the last sixth of the kernel. Here blocks 2p and 2p + 1 share the images
 // p, p + P, p + 2P, ... (P pairs) unevenly: of the J * ITY row passes of the pair's J images the even block takes a share
-// of kEvenShareNum / kEvenShareDen, in whole images plus the first row passes of one image that the two blocks split
+// of even_share / kEvenShareDen, in whole images plus the first row passes of one image that the two blocks split
 // (each takes it last; both run its column pass). 1024 images of 256 x 256: the even block transforms 4 1/4 images, the odd one 3 3/4: 101.6 -> 96.5 us.
 // Which row goes to which block does not change any value: the output is bit-identical to the equal split.
-// (kEvenShareNum / kEvenShareDen in kernels.h; measured here: 17/32 and 18/32 level, -5.3 us per layer, 19/32 -3 us)
+// (even_share / kEvenShareDen, see kernels.h; measured here: 17/32 and 18/32 level, -5.3 us per layer, 19/32 -3 us)
 
 template <int LOGX, int LOGY, bool SHARE>
 __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
-                                                          int nimg)
+                                                          int nimg, int even_share)
 {
     using G = Geo2D<LOGX, LOGY>;
     constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     if constexpr (SHARE) {
         const int pairs = gridDim.x / 2, pr = blockIdx.x >> 1, odd = blockIdx.x & 1;     // the host launches an even grid
         const int J = (nimg - pr + pairs - 1) / pairs;                                    // images of this pair
-        const int even_passes = (J * ITY * kEvenShareNum + kEvenShareDen / 2) / kEvenShareDen;
+        const int even_passes = (J * ITY * even_share + kEvenShareDen / 2) / kEvenShareDen;
         const int whole = even_passes / ITY, rest = even_passes % ITY;                    // of the even block
         step = pairs;
         split = rest != 0;
@@ -583,6 +584,22 @@ int cu_count()
     return v;
 }
 
+int even_share_parts()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return kEvenShareDen / 2;
+    int v = cached[dev & 63].load(std::memory_order_relaxed);
+    if (v > 0) return v;
+    hipDeviceProp_t prop;
+    v = kEvenShareDen / 2;
+    if (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount == 256 &&
+        std::string(prop.gcnArchName).rfind("gfx950", 0) == 0)
+        v = 17;
+    cached[dev & 63].store(v, std::memory_order_relaxed);
+    return v;
+}
+
 template <int LOGX, int LOGY>
 static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, int nimg, hipStream_t stream)
 {
@@ -592,7 +609,7 @@ static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* ou
     const int blocks = nimg < cu_count() ? nimg : cu_count();
     // uneven shares between the blocks of a pair: a full grid (one block per CU, so that block parity is XCD parity), at
     // least two images per block (128 x 128 images are a single row pass each and are shared in whole images only)
-    const bool share = inverse && blocks == cu_count() && blocks % 2 == 0 && nimg >= 2 * blocks;
+    const bool share = inverse && blocks == cu_count() && blocks % 2 == 0 && nimg >= 2 * blocks && even_share_parts() != kEvenShareDen / 2;
     static std::atomic<unsigned long long> served[3];
     const void* fn = !inverse ? reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>)
                      : share ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, true>)
@@ -600,10 +617,10 @@ static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* ou
     if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse ? (share ? 2 : 1) : 0]); e != hipSuccess) return e;
     if (share)
         hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, true>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, nimg);
+                           out, nimg, even_share_parts());
     else if (inverse)
         hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, false>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, nimg);
+                           out, nimg, kEvenShareDen / 2);
     else
         hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
                            out, nimg);

@@ -195,7 +195,8 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
 // with the input resident in the Infinity Cache).
 template <int LOGDX, int COLS>
 __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride_persistent_kernel(const float2* __restrict__ in,
-                                                                                     float2* __restrict__ out, int DY, long npanels)
+                                                                                     float2* __restrict__ out, int DY, long npanels,
+                                                                                     int even_share)
 {
     using G = GeoStride<LOGDX, COLS>;
     constexpr int DX = G::DX, L = G::L;
@@ -222,14 +223,15 @@ __global__ __launch_bounds__((GeoStride<LOGDX, COLS>::THREADS)) void ifft_stride
         }
     };
     cpx c[NIN];
-    // The odd XCDs of this GPU store about a fifth slower than the even ones, and workgroup b runs on XCD b mod 8: the
-    // blocks 2p and 2p + 1 share the panels p, p + pairs, p + 2 pairs, ... of their pair 17 : 15 instead of evenly (the
-    // even block takes the first ones), so that both end together. An odd grid keeps the even split.
+    // The odd XCDs of an MI355X store about a fifth slower than the even ones, and workgroup b runs on XCD b mod 8: the
+    // blocks 2p and 2p + 1 share the panels p, p + pairs, p + 2 pairs, ... of their pair even_share : 32 - even_share
+    // (17 : 15 there, 16 : 16 on other parts; the even block takes the first ones), so that both end together. An odd
+    // grid keeps the even split.
     long panel = blockIdx.x, step = gridDim.x, last = npanels;
     if ((gridDim.x & 1) == 0) {
         const long pairs = gridDim.x >> 1, pr = blockIdx.x >> 1;
         const long J = (npanels - pr + pairs - 1) / pairs;          // panels of this pair (pr < npanels: the grid is no larger)
-        const long even = (J * kEvenShareNum + kEvenShareDen / 2) / kEvenShareDen;
+        const long even = (J * even_share + kEvenShareDen / 2) / kEvenShareDen;
         step = pairs;
         panel = (blockIdx.x & 1) ? pr + pairs * even : pr;
         last = (blockIdx.x & 1) ? npanels : pr + pairs * even;
@@ -327,7 +329,7 @@ static hipError_t launch_stride_c(const float2* in, float2* out, int DY, long ns
         }
         const long resident = (long)occ * cu_count();
         const dim3 pgrid((unsigned)(blocks < resident ? blocks : resident));
-        if (INVERSE) hipLaunchKernelGGL((ifft_stride_persistent_kernel<LOGDX, COLS>), pgrid, block, G::LDS_BYTES, stream, in, out, DY, blocks);
+        if (INVERSE) hipLaunchKernelGGL((ifft_stride_persistent_kernel<LOGDX, COLS>), pgrid, block, G::LDS_BYTES, stream, in, out, DY, blocks, even_share_parts());
         else hipLaunchKernelGGL((fft_stride_persistent_kernel<LOGDX, COLS>), pgrid, block, G::LDS_BYTES, stream, in, out, DY, blocks);
         return hipGetLastError();
     }
