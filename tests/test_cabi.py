@@ -44,3 +44,33 @@ def test_codelets_on_cpu(tmp_path):
                    check=True)
     out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
     assert out.strip().endswith("OK"), out
+
+
+def test_cmake_package_builds_and_links(tmp_path):
+    """the CMake side of the integration: the top-level CMakeLists.txt builds libturbofno.so for gfx950 (library target
+    only), installs it with its package file, and a consumer that says find_package(turbofno) +
+    target_link_libraries(... turbofno::turbofno) builds and runs (no GPU needed: it only asks for the ABI version and a
+    size rule)"""
+    import shutil
+    import pytest
+    if not shutil.which("cmake") or not os.path.exists("/opt/rocm/lib/llvm/bin/clang++"):
+        pytest.skip("cmake or the ROCm clang is not installed")
+    build, prefix, cons = str(tmp_path / "build"), str(tmp_path / "prefix"), tmp_path / "consumer"
+    gen = ["-G", "Ninja"] if shutil.which("ninja") else []
+    run = lambda *cmd: subprocess.run(list(cmd), check=True, capture_output=True, text=True, timeout=900)
+    run("cmake", "-S", ROOT, "-B", build, *gen, "-DCMAKE_HIP_COMPILER=/opt/rocm/lib/llvm/bin/clang++", "-DTURBOFNO_BUILD_DRIVERS=OFF")
+    run("cmake", "--build", build, "-j", "8")
+    run("cmake", "--install", build, "--prefix", prefix)
+    L = ctypes.CDLL(os.path.join(prefix, "lib", "libturbofno.so"))
+    for n in declared_symbols():
+        assert hasattr(L, n), n
+    cons.mkdir()
+    (cons / "CMakeLists.txt").write_text("cmake_minimum_required(VERSION 3.21)\nproject(consumer LANGUAGES CXX)\n"
+                                         "find_package(turbofno REQUIRED)\nadd_executable(consumer main.cpp)\n"
+                                         "target_link_libraries(consumer PRIVATE turbofno::turbofno)\n")
+    (cons / "main.cpp").write_text('#include <turbofno.h>\n#include <cstdio>\nint main() { std::printf("%d %d\\n", '
+                                   'turbofno_abi_version(), turbofno_query_2d_algo(16, 256, 256, 64, 64, 0)); return 0; }\n')
+    run("cmake", "-S", str(cons), "-B", str(cons / "b"), "-Dturbofno_DIR=" + os.path.join(prefix, "lib", "cmake", "turbofno"))
+    run("cmake", "--build", str(cons / "b"))
+    out = run(str(cons / "b" / "consumer")).stdout.split()
+    assert out == ["2", "2"], out
