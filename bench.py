@@ -188,11 +188,22 @@ def main():
         y1 = torch.empty((128, 64, 256), dtype=torch.complex64, device=dev)
         # the clustered kernel of this shape exchanges partial products through caller-owned memory: attached here, as
         # the 1D executables do; without it the library runs the kernel that splits K inside one block
+        # A launch of this size takes the GPU less time than the Python binding takes to validate its operands, so the
+        # timed calls go to the C ABI directly (same entry point, arguments prepared once) and the host stays ahead.
+        tf.layer_1d(x1, W1, y=y1)                           # once through the checking binding
+        stream = torch.cuda.current_stream().cuda_stream
+        abi_args = (64, 1, 256, 128, 128, x1.data_ptr(), W1.data_ptr(), y1.data_ptr(), 1.0, 0.0, stream)
+
+        def layer_1d_abi():
+            rc = tf.lib().turbofno_layer_1d(*abi_args)
+            assert rc == 0, rc
         with tf.ExchangeBuffer() as exchange:
             kernel_1d = tf.query_1d_kernel(256, 64, 128, 128, compute_units=0, exchange_attached=True)
-            t1d = timed(lambda: tf.layer_1d(x1, W1, y=y1), 50)
+            timed(layer_1d_abi, 50)
+            exchange.status()                               # the first launches after the idle set-up may start ragged
+            t1d = timed(layer_1d_abi, 200)
             ran_out = exchange.status()
-        t1d_plain = timed(lambda: tf.layer_1d(x1, W1, y=y1), 50)
+        t1d_plain = timed(layer_1d_abi, 200)
         b1d = 8 * 64 * 256 * (128 + 128) + 8 * 128 * 128
         f1d = 8.0 * (64 * 64) * 128 * 128                      # real flops of the complex contraction
         large_hidden = {"workload": "1D bs=64 DY=256 K=128 N=128", "kernel": kernel_1d, "ms": round(t1d, 4),
