@@ -52,6 +52,12 @@ def test_large_grids_and_long_axes():
     assert tf.query_2d_algo(1, 512, 512, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(8, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
     assert tf.query_2d_algo(8, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
+    # 512 rows of up to 256: two interleaved parts per image on the whole-image kernels once there is enough data
+    assert tf.query_2d_algo(16, 512, 256, 32, 64) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(4, 512, 256, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(16, 512, 128, 32, 64) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(8, 512, 128, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(32, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
 
 
 def test_queries_answer_zero_for_arguments_the_calls_refuse():
@@ -60,6 +66,7 @@ def test_queries_answer_zero_for_arguments_the_calls_refuse():
     assert tf.query_1d_kernel(200, 4, 64, 8, CUS) == 0              # not a power of two
     assert tf.query_2d_algo(1, 200, 256, 16, 64) == 0
     assert tf.query_2d_algo(1, 512, 512, 16, 64, tf.ALGO_WHOLE_IMAGE) == 0
+    assert tf.query_2d_algo(1, 512, 256, 16, 64, tf.ALGO_WHOLE_IMAGE) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(1, 256, 256, 16, 60) == 0
     assert tf.query_2d_algo(1, 256, 256, 16, 64, 9) == 0
     # an explicit algorithm is returned as it is

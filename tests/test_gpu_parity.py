@@ -149,6 +149,12 @@ def test_stride_stages(DX, DY, nsig, tol):
     (1, 1024, 128, 8, 64, 3),
     (1, 512, 1024, 8, 128, 3),
     (5, 128, 128, 8, 64, 3),         # 20 row blocks of 32 rows over 40 images: several images per persistent block
+    (1, 512, 128, 8, 64, 2),         # whole-image path with DX above 256: two / four decimated parts of 256 rows per image,
+    (2, 512, 256, 16, 64, 2),        # summed over by the contraction (2 K or 4 K channels: one chunk, ...
+    (1, 1024, 256, 8, 64, 2),
+    (1, 1024, 128, 24, 128, 2),      # ... 96 channels in chunks of 32, ...
+    (3, 512, 256, 40, 64, 2),        # ... 80 = 32 + 32 + 16, ...
+    (1, 1024, 256, 72, 64, 2),       # ... 288 channels: nine chunks)
 ])
 def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     print("case layer_2d", bs, DX, DY, K, N, algo, flush=True)
@@ -199,8 +205,8 @@ def test_error_codes():
     with pytest.raises(tf.TurboFNOError) as e:
         tf.layer_1d(torch.zeros((8, 1, 2048), dtype=torch.complex64, device="cuda"), W)
     assert e.value.code == 2
-    x2 = torch.zeros((8, 1, 512, 128), dtype=torch.complex64, device="cuda")
-    with pytest.raises(tf.TurboFNOError) as e:                     # whole-image path exists for 128 / 256 only
+    x2 = torch.zeros((8, 1, 128, 512), dtype=torch.complex64, device="cuda")
+    with pytest.raises(tf.TurboFNOError) as e:                     # whole-image path: rows (DY) of 128 / 256 only
         tf.layer_2d(x2, W, algo=2)
     assert e.value.code == 2
 

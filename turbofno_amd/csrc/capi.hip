@@ -34,7 +34,10 @@ int log2_exact(long v)
 }
 
 bool length_built(int logD) { return logD >= 7 && logD <= 10; }          // 1D kernels and the X-axis kernels
-bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // whole-image 2D kernels
+bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // whole-image 2D kernels, one block per image
+// the whole-image path of the 2D layer also takes DX of 512 and 1024, as two or four decimated parts of 256 rows
+bool whole_image_built(int DX, int DY) { return (DY == 128 || DY == 256) && (DX == 128 || DX == 256 || DX == 512 || DX == 1024); }
+int image_parts(int DX) { return DX > 256 ? DX / 256 : 1; }
 
 int check_gemm_dims(long M, int N, int K)
 {
@@ -56,6 +59,12 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (algo != TURBOFNO_2D_AUTO) return algo;
+    if (DX == 512 && DY <= 256 && ((long)K + N) * bs >= (DY == 256 ? 640 : 1280)) {
+        // two decimated parts of 256 rows per image on the whole-image kernels: 3-24 % ahead of three stages from
+        // 160 MiB of input and output (84 shapes measured, bs 2-32; behind by up to 60 % on small problems). DX = 1024:
+        // the intermediates of three stages are a sixteenth of the data and the two paths are level.
+        return TURBOFNO_2D_WHOLE_IMAGE;
+    }
     if (DX > 256 || DY > 256) {
         // an image no longer fits one block's LDS: three stages. The axis that is transformed first is the one whose
         // truncation shrinks the intermediates most, i.e. the longer one (DY = 4 DX: half the time of the other order;
@@ -155,7 +164,7 @@ int turbofno_query_2d_algo(int bs, int DX, int DY, int K, int N, int algo)
     const int logDX = log2_exact(DX), logDY = log2_exact(DY);
     if (!length_built(logDX) || !length_built(logDY)) return 0;
     if (algo < TURBOFNO_2D_AUTO || algo > TURBOFNO_2D_ROWS_FIRST) return 0;
-    if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256)) return 0;
+    if (algo == TURBOFNO_2D_WHOLE_IMAGE && !whole_image_built(DX, DY)) return 0;
     return pick_algo(bs, DX, DY, K, N, algo);
 }
 
@@ -287,7 +296,7 @@ size_t turbofno_layer_2d_workspace_bytes(int bs, int DX, int DY, int K, int N, i
 {
     if (bs <= 0 || DX <= 0 || DY <= 0 || K <= 0 || N <= 0) return 0;
     if (pick_algo(bs, DX, DY, K, N, algo) == TURBOFNO_2D_WHOLE_IMAGE)
-        return align256((size_t)K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
+        return align256((size_t)image_parts(DX) * K * bs * 4096 * sizeof(float2)) + align256((size_t)N * bs * 4096 * sizeof(float2));
     const int kept_rows_of = pick_algo(bs, DX, DY, K, N, algo) == TURBOFNO_2D_ROWS_FIRST ? DX : DY;
     return align256((size_t)K * bs * 64 * kept_rows_of * sizeof(float2)) + align256((size_t)N * bs * 64 * kept_rows_of * sizeof(float2));
 }
@@ -309,8 +318,8 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
         return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: only lengths in {128, 256, 512, 1024} are built", DX, DY);
     if (algo != TURBOFNO_2D_AUTO && algo != TURBOFNO_2D_THREE_KERNEL && algo != TURBOFNO_2D_WHOLE_IMAGE && algo != TURBOFNO_2D_ROWS_FIRST)
         return fail(TURBOFNO_ERR_INVALID_ARG, "unknown algo %d", algo);
-    if (algo == TURBOFNO_2D_WHOLE_IMAGE && (DX > 256 || DY > 256))
-        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the whole-image path is built for lengths in {128, 256}", DX, DY);
+    if (algo == TURBOFNO_2D_WHOLE_IMAGE && !whole_image_built(DX, DY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the whole-image path is built for DY in {128, 256} and DX in {128, 256, 512, 1024}", DX, DY);
     const int a = pick_algo(bs, DX, DY, K, N, algo);
     const size_t need = turbofno_layer_2d_workspace_bytes(bs, DX, DY, K, N, a);
     if (!workspace || workspace_bytes < need)
@@ -320,10 +329,11 @@ static int layer_2d_on(int bs, int DX, int DY, int K, int N, const void* x, cons
     const float2 alpha = make_float2(alpha_re, alpha_im);
     char* ws = (char*)workspace;
     if (a == TURBOFNO_2D_WHOLE_IMAGE) {
+        const int parts = image_parts(DX);         // DX above 256: the parts of an image are channels of the contraction
         float2* spec = (float2*)ws;
-        float2* cspec = (float2*)(ws + align256((size_t)K * bs * 4096 * sizeof(float2)));
+        float2* cspec = (float2*)(ws + align256((size_t)parts * K * bs * 4096 * sizeof(float2)));
         if (int rc = hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, spec, K * bs, st), "fft2d_trunc launch")) return rc;
-        if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, K, alpha, make_float2(0.f, 0.f), st), "cgemm_modes launch")) return rc;
+        if (int rc = hip_status(tfno::launch_cgemm_modes(spec, (const float2*)W, cspec, (long)bs * 4096, N, parts * K, alpha, make_float2(0.f, 0.f), st, K), "cgemm_modes launch")) return rc;
         return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, cspec, (float2*)y, N * bs, st), "ifft2d_pad launch");
     }
     if (a == TURBOFNO_2D_ROWS_FIRST) {

@@ -131,11 +131,15 @@ hipError_t launch_ifft_stride(int logDX, const float2* in, float2* out, int DY, 
 hipError_t launch_fft_rows_trunc(int logDY, const float2* in, float2* out, int DX, long nimg, hipStream_t stream);
 hipError_t launch_ifft_rows_pad(int logDY, const float2* in, float2* out, int DX, long nimg, hipStream_t stream);
 
-// Whole-image 2D path (DX, DY in {128, 256}): truncated 2D forward transform per image, mode-space CGEMM
-// on the matrix cores, zero-padded 2D backward transform per image. nimg: the C ABI rejects counts beyond INT_MAX.
+// Whole-image 2D path (DY in {128, 256}; DX in {128, 256}, or 512 / 1024 as two / four decimated parts of 256 rows):
+// truncated 2D forward transform per image, mode-space CGEMM on the matrix cores, zero-padded 2D backward transform per
+// image. nimg: whole images; the C ABI rejects counts beyond INT_MAX. With R = DX / 256 > 1 parts, launch_fft2d_trunc
+// writes R * nimg spectra of 4096 modes (part r of image i at index r * nimg + i), to be summed over r: the contraction
+// does that when the parts are its channels r * K + k (launch_cgemm_modes with K = R * channels and w_period = channels);
+// launch_ifft2d_pad reads nimg spectra.
 hipError_t launch_fft2d_trunc(int logDX, int logDY, const float2* x, float2* spec, int nimg, hipStream_t stream);
 hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y, int nimg, hipStream_t stream);
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
-                              float2 beta, hipStream_t stream);
+                              float2 beta, hipStream_t stream, int w_period = 0);
 
 }  // namespace tfno

@@ -45,7 +45,11 @@ template <int LOGX, int LOGY> struct Geo2D {
     static_assert(LOGY == 7 || LOGY == 8, "rows of 128 or 256");
     static_assert(ITY >= 1 && COLT <= 1024, "unsupported image shape");
     // element offset of the lane's i-th sample from its first one
-    static __device__ __forceinline__ constexpr int sample_off(int i) { return PAIRED ? (i & 7) * 16 + (i >> 3) * (4 * DY) : 16 * i; }
+    // (logr: the rows of the image lie 2^logr rows of the array apart, see the decimated images below)
+    static __device__ __forceinline__ constexpr int sample_off(int i, int logr = 0)
+    {
+        return PAIRED ? (i & 7) * 16 + (i >> 3) * ((4 * DY) << logr) : 16 * i;
+    }
 };
 
 // First row (within one pass) of lane group g. The two groups that share an LDS cycle (one half wavefront) must
@@ -62,6 +66,29 @@ template <bool PAIRED> __device__ __forceinline__ int first_row_in_pass(int g)
         return (s & 3) + 8 * (s >> 2);
     }
 }
+
+// Decimated images (LOGR > 0): an image of R DX x DY, R = 2^LOGR, too long along X for one block, is handled as R parts
+// of DX x DY: part r holds the rows R j + r. Its transform along X splits exactly (one radix-R decimation in time step):
+//     X[p] = sum_{r<R} w_{R DX}^(r p) * DFT_DX(part r)[p],    p < 64
+// so the forward kernel transforms every part like an image of its own and multiplies its 64 x 64 modes by w^(r p); the
+// sum over r is a sum over "channels" and is done by the contraction that follows (channel r K + k, weight W[k]): the
+// parts are numbered r * nfull + image for that, nfull whole images. Backward, the R parts of an output image are
+// transformed from the one spectrum of the image, multiplied by conj(w^(r p)). Nothing but x, y and the 64 x 64 modes
+// ever leaves a CU, as for images of one block.
+template <int LOGX, int LOGR> __device__ __forceinline__ long first_array_row(long img, int nfull)
+{
+    if constexpr (LOGR == 0) return img << LOGX;
+    else {
+        const unsigned part = (unsigned)img / (unsigned)nfull, image = (unsigned)img - part * (unsigned)nfull;
+        return ((long)image << (LOGX + LOGR)) + part;
+    }
+}
+constexpr int kDecimationTwiddles = 64 * 4;      // complex elements: R <= 4 parts
+template <int LOGD> __device__ __forceinline__ void fill_decimation_twiddles(float2* tab, int tid, int nthreads)
+{
+    for (int e = tid; e < kDecimationTwiddles; e += nthreads)
+        tab[e] = kTwiddle1024[(((e >> 6) * (e & 63)) << (10 - LOGD)) & 1023];
+}
 }  // namespace
 
 // Forward image kernel: truncated 2D transform of one DX x DY image per block iteration.
@@ -72,12 +99,12 @@ template <bool PAIRED> __device__ __forceinline__ int first_row_in_pass(int g)
 // Each group keeps ONE row in flight: the loads of its next row are issued as soon as the first radix-4
 // stage has consumed the row registers, so they travel while the rest of the transform runs, across the
 // column pass and across image boundaries. Inter-pass twiddles live in LDS to stay within 128 VGPRs.
-template <int LOGX, int LOGY>
+template <int LOGX, int LOGY, int LOGR>
 __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
-                                                           int nimg)
+                                                           int nimg, int nfull)
 {
     using G = Geo2D<LOGX, LOGY>;
-    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
+    constexpr int DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x;
     const int gy = tid / LY, ty = tid % LY;            // row pass: group and lane
@@ -90,6 +117,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
     fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
     const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
+    float2* twsub = twtab_x + kTwLdsSize;              // decimated images: w^(r p) of the long axis, r < R, p < 64
+    if constexpr (LOGR > 0) fill_decimation_twiddles<LOGX + LOGR>(twsub, tid, 1024);
     __syncthreads();
 
     const int row0 = first_row_in_pass<G::PAIRED>(gy);
@@ -97,23 +126,24 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
     const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;
     const int tq = G::PAIRED ? (ty & 7) : ty;
     // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
-    const unsigned lane_off = (unsigned)(row0 * DY + ty);
+    const unsigned lane_off = (unsigned)(((row0 * DY) << LOGR) + ty);
     // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
     // next kernel re-reads, out of L2 / Infinity Cache
-    auto issue = [&](cpx (&dst)[16], long img, int it, unsigned off) {
-        const float2* base = x + (img * DX + G::RPP * it) * (long)DY;
+    auto issue = [&](cpx (&dst)[16], long array_row, int it, unsigned off) {
+        const float2* base = x + (array_row + ((G::RPP * it) << LOGR)) * (long)DY;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + (unsigned)G::sample_off(i)]);
+        for (int i = 0; i < 16; ++i) dst[i] = load_streaming(&base[off + (unsigned)G::sample_off(i, LOGR)]);
     };
 
     long img = blockIdx.x;
+    long img_row = first_array_row<LOGX, LOGR>(img < nimg ? img : 0, nfull);
     cpx v[16];
-    if (img < nimg) issue(v, img, 0, lane_off);
+    if (img < nimg) issue(v, img_row, 0, lane_off);
     for (; img < nimg; img += gridDim.x) {
         // look-ahead target: the next image's first rows; after the last image every lane group re-reads the
         // same row (row 0 of image 0, cache resident) so the loop stays branch free at no HBM cost
         const bool more = img + gridDim.x < nimg;
-        const long pre = more ? img + gridDim.x : 0;
+        const long pre_row = first_array_row<LOGX, LOGR>(more ? img + gridDim.x : 0, nfull);
         const unsigned pre_off = more ? lane_off : (unsigned)ty;
         // pass 1: rows (along Y). T[it][mm] = mode tq + 16 mm (paired rows: tq + 8 mm) of row trow + RPP it
         cpx T[ITY][MMY];
@@ -124,8 +154,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
                 fft16_stage1<-1>(v, bb);
                 // v is dead after the first radix-4 stage: its registers become the landing zone of the next row;
                 // the last pass already fetches the next image's first row
-                if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
-                else issue(v, pre, 0, pre_off);
+                if (it + 1 < ITY) issue(v, img_row, it + 1, lane_off);
+                else issue(v, pre_row, 0, pre_off);
                 fwd_pass1_lds_finish(bb, twrow_y, gg);
                 group_forward_finish<8>(gg, exch_y, ty, T[it]);
             } else {
@@ -139,8 +169,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
 #pragma unroll
                     for (int r = 0; r < 8; ++r) gg[r] = a8[r];
                 }
-                if (it + 1 < ITY) issue(v, img, it + 1, lane_off);
-                else issue(v, pre, 0, pre_off);
+                if (it + 1 < ITY) issue(v, img_row, it + 1, lane_off);
+                else issue(v, pre_row, 0, pre_off);
                 gg[8] = b8[0];
 #pragma unroll
                 for (int r = 1; r < 8; ++r) {
@@ -169,12 +199,21 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
             cpx gg[16], z[MMX];
             fwd_pass1_lds(c, twrow_x, gg);
             group_forward_finish<LOGX>(gg, exch_x, tx, z);
+            if constexpr (LOGR > 0) {
+                // part r of a decimated image: its modes enter the sum over the parts with w^(r p) of the long axis
+                const unsigned r = (unsigned)img / (unsigned)nfull;
+                if (r != 0) {
+#pragma unroll
+                    for (int mm = 0; mm < MMX; ++mm) z[mm] = cmul(z[mm], twsub[r * 64 + tx + LX * mm]);
+                }
+            }
             // lane order of the retained modes: element mm*COLT + q*LX + tx  <->  mode (p = tx + LX mm, q).
             // Written through as it is produced, so the end-of-kernel cache write-back has nothing left to flush
             float2* dst = spec + img * 4096;
 #pragma unroll
             for (int mm = 0; mm < MMX; ++mm) store_streaming(dst + tid + G::COLT * mm, z[mm]);
         }
+        img_row = pre_row;
     }
 }
 
@@ -192,12 +231,12 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
 // Which row goes to which block does not change any value: the output is bit-identical to the equal split.
 // (even_share / kEvenShareDen, see kernels.h; measured here: 17/32 and 18/32 level, -5.3 us per layer, 19/32 -3 us)
 
-template <int LOGX, int LOGY, bool SHARE>
+template <int LOGX, int LOGY, bool SHARE, int LOGR>
 __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restrict__ spec, float2* __restrict__ y,
-                                                          int nimg, int even_share)
+                                                          int nimg, int even_share, int nfull)
 {
     using G = Geo2D<LOGX, LOGY>;
-    constexpr int DX = G::DX, DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
+    constexpr int DY = G::DY, LX = G::LX, LY = G::LY, ITY = G::ITY, MMY = G::MMY, MMX = G::MMX;
     extern __shared__ float2 lds[];
     const int tid = threadIdx.x;
     const int gy = tid / LY, ty = tid % LY;
@@ -210,13 +249,17 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
     const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
+    float2* twsub = twtab_x + kTwLdsSize;
+    if constexpr (LOGR > 0) fill_decimation_twiddles<LOGX + LOGR>(twsub, tid, 1024);
     __syncthreads();
 
     const int row0 = first_row_in_pass<G::PAIRED>(gy);
     const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;      // row whose modes the lane takes from the tile
     const int tq = G::PAIRED ? (ty & 7) : ty;
-    const unsigned lane_off = (unsigned)(row0 * DY + ty);
+    const unsigned lane_off = (unsigned)(((row0 * DY) << LOGR) + ty);
     const bool col_thread = tid < G::COLT;
+    // part r of a decimated image is transformed from the spectrum of the whole image
+    auto spectrum_of = [&](long img) { return spec + (LOGR > 0 ? (long)((unsigned)img % (unsigned)nfull) : img) * 4096; };
 
     // The block transforms `count` images, image_at(k) for k < count; of its last one, if `split`, only the row passes
     // [pass0, pass1). Without SHARE: every block the images blockIdx.x, + gridDim.x, ... in full.
@@ -245,7 +288,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 
     cpx c[MMX];
     if (count > 0 && col_thread) {
-        const float2* src = spec + image_at(0) * 4096;
+        const float2* src = spectrum_of(image_at(0));
 #pragma unroll
         for (int mm = 0; mm < MMX; ++mm) c[mm] = src[tid + G::COLT * mm];
     }
@@ -256,6 +299,13 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
         const int it0 = partial ? pass0 : 0, it1 = partial ? pass1 : ITY;
         // pass 1: columns (p -> x) of column q = gx
         cpx u[16];
+        if constexpr (LOGR > 0) {
+            const unsigned r = (unsigned)img / (unsigned)nfull;
+            if (r != 0 && col_thread) {
+#pragma unroll
+                for (int mm = 0; mm < MMX; ++mm) c[mm] = cmulc(c[mm], twsub[r * 64 + tx + LX * mm]);
+            }
+        }
         if (col_thread) group_backward_lds<LOGX>(c, twrow_x, exch_x, tx, u);
         // the exchange regions alias the tile: every wave must be done with them before the tile is written
         __syncthreads();
@@ -263,7 +313,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 #pragma unroll
             for (int i = 0; i < 16; ++i) lds[(tx + LX * i) * TPITCH + gx] = u[i];
             // next image's spectrum (for the last image: a harmless re-read of its own 32 KiB)
-            const float2* src = spec + pre * 4096;
+            const float2* src = spectrum_of(pre);
 #pragma unroll
             for (int mm = 0; mm < MMX; ++mm) c[mm] = src[tid + G::COLT * mm];
         }
@@ -284,9 +334,10 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
             cpx yv[16];
             if constexpr (G::PAIRED) rows128_backward(cc[it], twrow_y, exch_y, ty, yv);
             else group_backward_lds<8>(cc[it], twrow_y, exch_y, ty, yv);
-            float2* dst = y + (img * DX + G::RPP * it) * (long)DY;   // uniform base + lane offset + immediates
+            // uniform base + lane offset + immediates
+            float2* dst = y + (first_array_row<LOGX, LOGR>(img, nfull) + ((G::RPP * it) << LOGR)) * (long)DY;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + G::sample_off(i), yv[i]);
+            for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + G::sample_off(i, LOGR), yv[i]);
         }
     }
 }
@@ -307,6 +358,8 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
 // matrix work of the next ones.
 //   NG    = channel groups of four per chunk that can hold data (4, 8, 12, 16 for K <= 16, 32, 48, 64): a template
 //           parameter so that the loops stay unrolled and no loads or matrix work are spent on zero padding;
+//   Kw    = period of W along the contraction: channel k is weighted with W[k mod Kw + n Kw] (Kw = K: the plain product;
+//           Kw = K / R: the R parts of decimated images, see above, share the weights of their image's channel);
 //   MULTI = K > 64: chunks of 4 NG = 32 channels with the twelve accumulator tiles of a wave kept across them
 //           (125 registers; 64-channel chunks would spill); otherwise one chunk and transient accumulators.
 // ---------------------------------------------------------------------------------------------
@@ -325,7 +378,8 @@ constexpr int kW3Row = 80, kW3Group = 4 * kW3Row + 1, kW3Plane = (GEMM_KC / 4) *
 template <int NG, bool MULTI>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float2* __restrict__ A,
                                                                      const float2* __restrict__ W, float2* __restrict__ C,
-                                                                     long Mtot, int N, int K, float2 alpha, float2 beta)
+                                                                     long Mtot, int N, int K, float2 alpha, float2 beta,
+                                                                     int Kw)
 {
     extern __shared__ float sW[];                     // 3 * kW3Plane floats
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
@@ -371,7 +425,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_kernel(const float
             for (int u = 0; u < WPT; ++u) {
                 const int idx = tid + u * BUILDERS;
                 const int k = idx % KCH, n = idx / KCH;
-                wv[u] = (k < kn) ? W[(kc + k) + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+                wv[u] = (k < kn) ? W[(kc + k) % Kw + (long)(n0 + n) * Kw] : make_float2(0.f, 0.f);
             }
 #pragma unroll
             for (int u = 0; u < WPT; ++u) {
@@ -424,7 +478,7 @@ template <int NG>
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(const float2* __restrict__ A,
                                                                                 const float2* __restrict__ W,
                                                                                 float2* __restrict__ C, long Mtot, int N, int K,
-                                                                                float2 alpha, long nblocks)
+                                                                                float2 alpha, long nblocks, int Kw)
 {
     extern __shared__ float sW[];                     // 3 * kW3Plane floats
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, kq = lane >> 4;
@@ -448,7 +502,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_kernel(
         for (int u = 0; u < WPT; ++u) {
             const int idx = tid + u * GEMM_THREADS;
             const int k = idx % GEMM_KC, n = idx / GEMM_KC;
-            wv[u] = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+            wv[u] = (k < K) ? W[k % Kw + (long)(n0 + n) * Kw] : make_float2(0.f, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < WPT; ++u) {
@@ -504,7 +558,7 @@ constexpr int kW3WidePlane = (GEMM_KMAX / 4) * kW3Group;
 __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_wide_kernel(const float2* __restrict__ A,
                                                                                      const float2* __restrict__ W,
                                                                                      float2* __restrict__ C, long Mtot, int N, int K,
-                                                                                     float2 alpha, long nblocks)
+                                                                                     float2 alpha, long nblocks, int Kw)
 {
     extern __shared__ float sW[];                     // 3 * kW3WidePlane floats
     constexpr int NG = 8;                             // channel groups per chunk
@@ -526,7 +580,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void cgemm_modes3m_persistent_wide_ke
     for (int g = 0; g < NG; ++g) bv[g] = strip_elem(block_of(v), 0, g);
     for (int idx = tid; idx < GEMM_KMAX * 64; idx += GEMM_THREADS) {
         const int k = idx % GEMM_KMAX, n = idx / GEMM_KMAX;
-        const float2 w = (k < K) ? W[k + (long)(n0 + n) * K] : make_float2(0.f, 0.f);
+        const float2 w = (k < K) ? W[k % Kw + (long)(n0 + n) * Kw] : make_float2(0.f, 0.f);
         const float c = w.x * alpha.x - w.y * alpha.y, d = w.x * alpha.y + w.y * alpha.x;
         float* dstw = &sW[(k >> 2) * kW3Group + (k & 3) * kW3Row + n];
         dstw[0] = c;
@@ -600,10 +654,13 @@ int even_share_parts()
     return v;
 }
 
-template <int LOGX, int LOGY>
-static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, int nimg, hipStream_t stream)
+template <int LOGX, int LOGY, int LOGR>
+static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* out, int nfull, hipStream_t stream)
 {
     using G = Geo2D<LOGX, LOGY>;
+    if (nfull <= 0 || nfull > (0x7fffffff >> LOGR)) return hipErrorInvalidValue;
+    const int nimg = nfull << LOGR;                    // images of one block each: the 2^LOGR parts of every image
+    const size_t lds_bytes = G::LDS_BYTES + (LOGR > 0 ? sizeof(float2) * kDecimationTwiddles : 0);
     // persistent blocks: at most as many as fit at once (LDS allows one or two 1024-thread blocks per CU,
     // the thread count exactly one)
     const int blocks = nimg < cu_count() ? nimg : cu_count();
@@ -611,29 +668,34 @@ static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* ou
     // least two images per block (128 x 128 images are a single row pass each and are shared in whole images only)
     const bool share = inverse && blocks == cu_count() && blocks % 2 == 0 && nimg >= 2 * blocks && even_share_parts() != kEvenShareDen / 2;
     static std::atomic<unsigned long long> served[3];
-    const void* fn = !inverse ? reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY>)
-                     : share ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, true>)
-                             : reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, false>);
-    if (hipError_t e = allow_dynamic_lds(fn, G::LDS_BYTES, served[inverse ? (share ? 2 : 1) : 0]); e != hipSuccess) return e;
+    const void* fn = !inverse ? reinterpret_cast<const void*>(fft2d_trunc_kernel<LOGX, LOGY, LOGR>)
+                     : share ? reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, true, LOGR>)
+                             : reinterpret_cast<const void*>(ifft2d_pad_kernel<LOGX, LOGY, false, LOGR>);
+    if (hipError_t e = allow_dynamic_lds(fn, lds_bytes, served[inverse ? (share ? 2 : 1) : 0]); e != hipSuccess) return e;
     if (share)
-        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, true>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, nimg, even_share_parts());
+        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, true, LOGR>), dim3((unsigned)blocks), dim3(1024), lds_bytes, stream, in,
+                           out, nimg, even_share_parts(), nfull);
     else if (inverse)
-        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, false>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, nimg, kEvenShareDen / 2);
+        hipLaunchKernelGGL((ifft2d_pad_kernel<LOGX, LOGY, false, LOGR>), dim3((unsigned)blocks), dim3(1024), lds_bytes, stream, in,
+                           out, nimg, kEvenShareDen / 2, nfull);
     else
-        hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY>), dim3((unsigned)blocks), dim3(1024), G::LDS_BYTES, stream, in,
-                           out, nimg);
+        hipLaunchKernelGGL((fft2d_trunc_kernel<LOGX, LOGY, LOGR>), dim3((unsigned)blocks), dim3(1024), lds_bytes, stream, in,
+                           out, nimg, nfull);
     return hipGetLastError();
 }
 
+// DX of 512 or 1024: two or four decimated parts of 256 rows each
 static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, const float2* in, float2* out, int nimg,
                                         hipStream_t stream)
 {
-    if (logDX == 8 && logDY == 8) return launch_image_kernel<8, 8>(inverse, in, out, nimg, stream);
-    if (logDX == 8 && logDY == 7) return launch_image_kernel<8, 7>(inverse, in, out, nimg, stream);
-    if (logDX == 7 && logDY == 8) return launch_image_kernel<7, 8>(inverse, in, out, nimg, stream);
-    if (logDX == 7 && logDY == 7) return launch_image_kernel<7, 7>(inverse, in, out, nimg, stream);
+    if (logDX == 8 && logDY == 8) return launch_image_kernel<8, 8, 0>(inverse, in, out, nimg, stream);
+    if (logDX == 8 && logDY == 7) return launch_image_kernel<8, 7, 0>(inverse, in, out, nimg, stream);
+    if (logDX == 7 && logDY == 8) return launch_image_kernel<7, 8, 0>(inverse, in, out, nimg, stream);
+    if (logDX == 7 && logDY == 7) return launch_image_kernel<7, 7, 0>(inverse, in, out, nimg, stream);
+    if (logDX == 9 && logDY == 8) return launch_image_kernel<8, 8, 1>(inverse, in, out, nimg, stream);
+    if (logDX == 9 && logDY == 7) return launch_image_kernel<8, 7, 1>(inverse, in, out, nimg, stream);
+    if (logDX == 10 && logDY == 8) return launch_image_kernel<8, 8, 2>(inverse, in, out, nimg, stream);
+    if (logDX == 10 && logDY == 7) return launch_image_kernel<8, 7, 2>(inverse, in, out, nimg, stream);
     return hipErrorInvalidValue;
 }
 
@@ -648,9 +710,11 @@ hipError_t launch_ifft2d_pad(int logDX, int logDY, const float2* spec, float2* y
 }
 
 hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long Mtot, int N, int K, float2 alpha,
-                              float2 beta, hipStream_t stream)
+                              float2 beta, hipStream_t stream, int w_period)
 {
     if (Mtot % 16 != 0 || Mtot <= 0 || Mtot >= (1L << 27) || N % 64 != 0 || K % 8 != 0) return hipErrorInvalidValue;
+    const int Kw = w_period > 0 ? w_period : K;
+    if (K % Kw != 0) return hipErrorInvalidValue;
     dim3 grid((unsigned)((Mtot + GEMM_MBLOCK - 1) / GEMM_MBLOCK), (unsigned)(N / 64), 1);
     constexpr size_t lds_bytes = sizeof(float) * 3 * kW3Plane;      // 61,632 B: above the static limit
     auto launch = [&](auto ng_const, auto multi_const) -> hipError_t {
@@ -661,7 +725,7 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
             e != hipSuccess)
             return e;
         hipLaunchKernelGGL((cgemm_modes3m_kernel<NG, MULTI>), grid, dim3(GEMM_THREADS), lds_bytes, stream, A, W, C, Mtot, N, K,
-                           alpha, beta);
+                           alpha, beta, Kw);
         return hipGetLastError();
     };
     // several column blocks per CU, one chunk: persistent blocks, one per CU (and n tile)
@@ -680,7 +744,7 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         if (g >= 8) g -= g % 8;                                  // whole groups of eight: every XCD the same share
         if (g < 1) g = 1;
         hipLaunchKernelGGL((cgemm_modes3m_persistent_kernel<NG>), dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), lds_bytes,
-                           stream, A, W, C, Mtot, N, K, alpha, nblocks);
+                           stream, A, W, C, Mtot, N, K, alpha, nblocks, Kw);
         return hipGetLastError();
     };
     // from two column blocks per CU (K = N = 64: M = 131,072 40 -> 37 us, 262,144 75 -> 64, 524,288 164 -> 133; below that
@@ -707,7 +771,7 @@ hipError_t launch_cgemm_modes(const float2* A, const float2* W, float2* C, long 
         if (g < 1) g = 1;
         if (g > (long)grid.x) g = grid.x;
         hipLaunchKernelGGL(cgemm_modes3m_persistent_wide_kernel, dim3((unsigned)g, grid.y, 1), dim3(GEMM_THREADS), wide_lds, stream, A,
-                           W, C, Mtot, N, K, alpha, (long)grid.x);
+                           W, C, Mtot, N, K, alpha, (long)grid.x, Kw);
         return hipGetLastError();
     }
     if (K <= 16) return launch(std::integral_constant<int, 4>{}, std::false_type{});
