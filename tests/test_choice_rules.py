@@ -47,17 +47,26 @@ def test_large_grids_and_long_axes():
     assert tf.query_1d_kernel(128, 4096, 64, 64, CUS) == 5
     assert tf.query_1d_kernel(128, 4096, 128, 128, CUS) == 8
     assert tf.query_1d_kernel(512, 4096, 64, 32, CUS) == 1
-    # axes above 256: three stages, the longer axis (or, for squares with enough images, the contiguous one) first
-    assert tf.query_2d_algo(16, 512, 512, 32, 64) == tf.ALGO_ROWS_FIRST
+    # axes above 256, small problems: three stages, the longer axis (or, for squares with enough images, the contiguous
+    # one) first
+    assert tf.query_2d_algo(2, 512, 512, 64, 64) == tf.ALGO_ROWS_FIRST
     assert tf.query_2d_algo(1, 512, 512, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(8, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
     assert tf.query_2d_algo(8, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
-    # 512 rows of up to 256: two interleaved parts per image on the whole-image kernels once there is enough data
+    assert tf.query_2d_algo(2, 1024, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
+    # large ones: the whole-image kernels (512 / 1024 rows as interleaved parts of 256, long rows with 32 / 64 lanes)
+    assert tf.query_2d_algo(16, 512, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(4, 512, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE            # 768 MiB
+    assert tf.query_2d_algo(4, 512, 512, 16, 64) == tf.ALGO_THREE_KERNEL           # 640 MiB
     assert tf.query_2d_algo(16, 512, 256, 32, 64) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(4, 512, 256, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(16, 512, 128, 32, 64) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(8, 512, 128, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(16, 256, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(32, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(16, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
+    assert tf.query_2d_algo(16, 256, 1024, 32, 128) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(16, 1024, 1024, 32, 64) == tf.ALGO_WHOLE_IMAGE
 
 
 def test_queries_answer_zero_for_arguments_the_calls_refuse():
@@ -65,9 +74,9 @@ def test_queries_answer_zero_for_arguments_the_calls_refuse():
     assert tf.query_1d_kernel(2048, 4, 64, 8, CUS) == 0             # no kernel of that length
     assert tf.query_1d_kernel(200, 4, 64, 8, CUS) == 0              # not a power of two
     assert tf.query_2d_algo(1, 200, 256, 16, 64) == 0
-    assert tf.query_2d_algo(1, 512, 512, 16, 64, tf.ALGO_WHOLE_IMAGE) == 0
-    assert tf.query_2d_algo(1, 512, 256, 16, 64, tf.ALGO_WHOLE_IMAGE) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(1, 2048, 512, 16, 64, tf.ALGO_WHOLE_IMAGE) == 0
     assert tf.query_2d_algo(1, 256, 256, 16, 60) == 0
     assert tf.query_2d_algo(1, 256, 256, 16, 64, 9) == 0
     # an explicit algorithm is returned as it is
     assert tf.query_2d_algo(1, 256, 256, 16, 64, tf.ALGO_WHOLE_IMAGE) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(1, 512, 1024, 16, 64, tf.ALGO_WHOLE_IMAGE) == tf.ALGO_WHOLE_IMAGE

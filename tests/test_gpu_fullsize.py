@@ -134,15 +134,19 @@ def test_config4_small_batches_against_oracle(bs, D, K, tol):
 
 
 @pytest.mark.parametrize("bs,DX,DY,K,N,algo", [
-    (4, 512, 512, 32, 64, 0),        # whole rows first by size: 2048 row blocks of 32 rows on at most 768 persistent blocks
+    (4, 512, 512, 32, 64, 0),        # 768 MiB of 512 x 512: the whole-image kernels by size (768 + 1024 parts of 256 x 512)
+    (4, 512, 512, 32, 64, 3),        # whole rows first: 2048 row blocks of 32 rows on at most 768 persistent blocks
     (4, 256, 1024, 32, 64, 0),       # DY > DX: whole rows first, eight batches of rows per block
     (4, 1024, 256, 32, 64, 0),       # DX > DY: X axis first
     (6, 512, 512, 24, 128, 1),
     (6, 512, 512, 24, 128, 3),
+    (6, 512, 256, 24, 128, 2),       # whole-image kernels, several parts per persistent block: two parts per image, ...
+    (3, 1024, 512, 24, 64, 2),       # ... four parts and rows of 512, ...
+    (5, 256, 1024, 40, 128, 2),      # ... rows of 1024
 ])
 def test_large_images_against_oracle_slices(bs, DX, DY, K, N, algo, tol):
-    """lengths above 256 at sizes that run the persistent loops of the X-axis kernels and of the row kernels several times
-    per block; first and last batch element against the oracle"""
+    """lengths above 256 at sizes that run the persistent loops of the X-axis kernels, of the row kernels and of the
+    whole-image kernels several times per block; first and last batch element against the oracle"""
     print("large images", bs, DX, DY, K, N, "algo", algo, flush=True)
     x_h, W_h = workloads.uniform_2d(950 + bs + DX + K + algo, bs, DX, DY, K, N)
     y = tf.layer_2d(torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda(), alpha=0.5 - 1j, algo=algo)

@@ -155,6 +155,14 @@ def test_stride_stages(DX, DY, nsig, tol):
     (1, 1024, 128, 24, 128, 2),      # ... 96 channels in chunks of 32, ...
     (3, 512, 256, 40, 64, 2),        # ... 80 = 32 + 32 + 16, ...
     (1, 1024, 256, 72, 64, 2),       # ... 288 channels: nine chunks)
+    (1, 128, 512, 8, 64, 2),         # whole-image path with rows of 512 / 1024: 32 / 64 lanes per row
+    (1, 256, 512, 16, 64, 2),
+    (2, 128, 1024, 8, 64, 2),
+    (1, 256, 1024, 24, 128, 2),
+    (1, 512, 512, 8, 64, 2),         # both: long rows and interleaved parts
+    (1, 1024, 512, 8, 64, 2),
+    (1, 512, 1024, 40, 64, 2),
+    (1, 1024, 1024, 8, 64, 2),
 ])
 def test_layer_2d(bs, DX, DY, K, N, algo, tol):
     print("case layer_2d", bs, DX, DY, K, N, algo, flush=True)
@@ -205,8 +213,8 @@ def test_error_codes():
     with pytest.raises(tf.TurboFNOError) as e:
         tf.layer_1d(torch.zeros((8, 1, 2048), dtype=torch.complex64, device="cuda"), W)
     assert e.value.code == 2
-    x2 = torch.zeros((8, 1, 128, 512), dtype=torch.complex64, device="cuda")
-    with pytest.raises(tf.TurboFNOError) as e:                     # whole-image path: rows (DY) of 128 / 256 only
+    x2 = torch.zeros((8, 1, 2048, 128), dtype=torch.complex64, device="cuda")
+    with pytest.raises(tf.TurboFNOError) as e:                     # no 2D kernel of that length, whatever the algorithm
         tf.layer_2d(x2, W, algo=2)
     assert e.value.code == 2
 

@@ -36,7 +36,7 @@ int log2_exact(long v)
 bool length_built(int logD) { return logD >= 7 && logD <= 10; }          // 1D kernels and the X-axis kernels
 bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // whole-image 2D kernels, one block per image
 // the whole-image path of the 2D layer also takes DX of 512 and 1024, as two or four decimated parts of 256 rows
-bool whole_image_built(int DX, int DY) { return (DY == 128 || DY == 256) && (DX == 128 || DX == 256 || DX == 512 || DX == 1024); }
+bool whole_image_built(int DX, int DY) { return length_built(log2_exact(DX)) && length_built(log2_exact(DY)); }
 int image_parts(int DX) { return DX > 256 ? DX / 256 : 1; }
 
 int check_gemm_dims(long M, int N, int K)
@@ -59,14 +59,23 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
 {
     if (algo != TURBOFNO_2D_AUTO) return algo;
-    if (DX == 512 && DY <= 256 && ((long)K + N) * bs >= (DY == 256 ? 640 : 1280)) {
-        // two decimated parts of 256 rows per image on the whole-image kernels: 3-24 % ahead of three stages from
-        // 160 MiB of input and output (84 shapes measured, bs 2-32; behind by up to 60 % on small problems). DX = 1024:
-        // the intermediates of three stages are a sixteenth of the data and the two paths are level.
-        return TURBOFNO_2D_WHOLE_IMAGE;
+    if (DX > 256 || DY > 256) {
+        // Long axes on the whole-image kernels (512 / 1024 rows as interleaved parts of 256, rows of 512 / 1024 with 32 /
+        // 64 lanes each): x and y move once and nothing but 64 x 64 modes in between, against intermediates of 1/8 (length
+        // 512) or 1/16 (1024) of the data, twice over, for three stages. Measured on MI355X (324 shapes, bs 1-32, all three
+        // paths back to back), with `mib` the input and output in MiB: DX = 512 with rows up to 256 ahead by 3-24 % from
+        // 640 MiB, rows of 512 by 1-22 % from 768 MiB (3 GiB of 512 x 512: 752 -> 608 us); rows of 1024 level with whole
+        // rows first (within 5 %) except for the large problems below (8-16 %); behind by up to 2x on small problems.
+        const long mib = ((long)K + N) * bs * DX * DY >> 17;
+        bool whole;
+        if (DY <= 256) whole = DX == 512 && mib >= 640;
+        else if (DY == 512) whole = mib >= 768;
+        else whole = (DX == 256 && N >= 128 && mib >= 4608) || (DX == 512 && mib >= 4608 && (N >= 128 || bs >= 16)) ||
+                     (DX == 1024 && mib >= 9216);
+        if (whole) return TURBOFNO_2D_WHOLE_IMAGE;
     }
     if (DX > 256 || DY > 256) {
-        // an image no longer fits one block's LDS: three stages. The axis that is transformed first is the one whose
+        // otherwise three stages. The axis that is transformed first is the one whose
         // truncation shrinks the intermediates most, i.e. the longer one (DY = 4 DX: half the time of the other order;
         // DX = 4 DY: the reverse). Square images: whole rows first (9-18 % ahead) unless the grid is small.
         if (DY != DX) return DY > DX ? TURBOFNO_2D_ROWS_FIRST : TURBOFNO_2D_THREE_KERNEL;

@@ -238,9 +238,10 @@ constexpr int kTwLdsPitch = 18;
 constexpr int kTwLdsSize = 16 * kTwLdsPitch;   // complex elements
 
 #ifdef __HIPCC__
-template <int LOGD> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
+template <int LOGD, int ROWS = 16> TFNO_DEV void fill_lds_twiddles(cpx* tab, int tid, int nthreads)
 {
-    for (int e = tid; e < 256; e += nthreads) {      // all 16 lane rows (groups of fewer lanes use the first ones)
+    // all 16 lane rows (groups of fewer lanes use the first ones); ROWS = 32 / 64 for the lane groups of lengths 512 / 1024
+    for (int e = tid; e < 16 * ROWS; e += nthreads) {
         const int t = e >> 4, r = e & 15;
         tab[t * kTwLdsPitch + r] = kTwiddle1024[((t * r) << (10 - LOGD)) & 1023];
     }
@@ -354,12 +355,11 @@ template <int L> TFNO_DEV void wide_forward_outer(const cpx* swap, int es, int l
 // lane t1 + (L/4) t2, slot r: the caller parks it at wide_back_index<L>(l, 4 ri + t2) of a pitch-17 array [L][17] (after
 // every lane has read C, which may live in the same array) and each lane reads its e[r] back from row t. 16 + 16 + 16
 // exchange accesses and ~110 flops per lane instead of 64 reads and ~290 flops for the direct sums.
-template <int L> TFNO_DEV void wide_backward_partial(const cpx* c64, int es, int l, cpx (&part)[16])
+template <int L>
+TFNO_DEV void wide_backward_partial_tw(const cpx* c64, int es, int l, cpx w1, cpx w2, cpx w3, cpx (&part)[16])
 {
     constexpr int Q = L / 4;
-    const int t1 = l % Q, rq = l / Q;
-    const cpx w1 = kTwiddle1024[(t1 * (1024 / L)) & 1023], w2 = kTwiddle1024[(2 * t1 * (1024 / L)) & 1023],
-              w3 = kTwiddle1024[(3 * t1 * (1024 / L)) & 1023];
+    const int rq = l / Q;
 #pragma unroll
     for (int ri = 0; ri < 4; ++ri) {
         const int r = rq + 4 * ri;
@@ -372,6 +372,12 @@ template <int L> TFNO_DEV void wide_backward_partial(const cpx* c64, int es, int
         part[4 * ri + 2] = csub(s02, s13);
         part[4 * ri + 3] = csub(m02, im13);
     }
+}
+template <int L> TFNO_DEV void wide_backward_partial(const cpx* c64, int es, int l, cpx (&part)[16])
+{
+    const int t1 = l % (L / 4);
+    wide_backward_partial_tw<L>(c64, es, l, kTwiddle1024[(t1 * (1024 / L)) & 1023], kTwiddle1024[(2 * t1 * (1024 / L)) & 1023],
+                                kTwiddle1024[(3 * t1 * (1024 / L)) & 1023], part);
 }
 template <int L> TFNO_DEV constexpr int wide_back_index(int l, int k)
 {

@@ -188,6 +188,60 @@ TFNO_DEV void rows128_backward(const cpx (&c)[8], const TW& twrow, cpx* exch, in
     for (int i = 0; i < 8; ++i) { y[i] = a[i]; y[8 + i] = b[i]; }
 }
 
+// Rows of 512 / 1024 in the whole-image kernels: a group of L = 32 / 64 lanes owns one row, lane t holds samples t + L i.
+// The scheme of the wide_* codelets, with every twiddle taken from LDS (a global load inside the row loop would queue
+// behind the loads of the next row, which are in flight all the time): twrow = the lane's row of the first-pass table,
+// wsm[e] = w_L^e, e < L.
+// g[]: first-pass results, already twiddled. Lane t = A r + a (A = L / 16) finishes the modes r + 16 (a + A j), j < 64 / L,
+// in out[j]: for one j the lanes of a group hold L consecutive modes, so that they can be written to one row of a tile
+// without bank conflicts (the map of the 1D kernels, wide_mode, puts lanes 32 modes apart).
+template <int L> TFNO_DEV constexpr int wide_rows_mode(int t, int j) { return t / (L / 16) + 16 * (t % (L / 16) + (L / 16) * j); }
+template <int L>
+TFNO_DEV void wide_rows_forward_finish(const cpx (&g)[16], cpx* exch, const cpx* wsm, int t, cpx (&out)[64 / L])
+{
+    constexpr int A = L / 16, MM = 64 / L;
+    const int r = t / A, a = t % A;
+    wave_lds_fence();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) exch[t * 17 + k] = g[k];
+    wave_lds_fence();
+    cpx inner[4];
+    wide_forward_inner<L>(exch, 1, t, inner);
+    wave_lds_fence();                                // every lane of the group has read the first exchange
+#pragma unroll
+    for (int c = 0; c < 4; ++c) exch[wide_swap_index<L>(r, c, a)] = inner[c];
+    wave_lds_fence();
+#pragma unroll
+    for (int j = 0; j < MM; ++j) {
+        const int c = a + A * j;
+        cpx acc = exch[wide_swap_index<L>(r, c, 0)];
+#pragma unroll
+        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[wide_swap_index<L>(r, c, ap)], wsm[(ap * c) % L]);
+        out[j] = acc;
+    }
+}
+
+// c[mm] = mode t + L mm of the row. On return y[i] = sample t + L i.
+template <int L>
+TFNO_DEV void wide_rows_backward(const cpx (&c)[64 / L], const cpx* twrow, const cpx* wsm, cpx* exch, int t, cpx (&y)[16])
+{
+    wave_lds_fence();
+#pragma unroll
+    for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
+    wave_lds_fence();
+    cpx part[16];
+    const int t1 = t % (L / 4);
+    wide_backward_partial_tw<L>(exch, 1, t, wsm[t1], wsm[2 * t1], wsm[3 * t1], part);
+    wave_lds_fence();                                // every lane of the group has read the 64 modes
+#pragma unroll
+    for (int k = 0; k < 16; ++k) exch[wide_back_index<L>(t, k)] = part[k];
+    wave_lds_fence();
+    cpx e[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+    inv_pass2_lds(e, twrow, y);
+}
+
 // The same pairing for the 1D kernels, with the twiddles in registers (tw[r] = w_128^(t r), t < 16): a 16-lane group
 // transforms two signals; v[0..7] / v[8..15] are samples t + 16 i of signal A / signal B. On return out[c] is mode
 // (t & 7) + 8 c of signal (t >> 3): the lane-to-mode mapping of an 8-lane group per signal, so callers index their

@@ -32,23 +32,37 @@ constexpr int EXCH_ELEMS = 1024 * 17;            // exchange regions of all lane
 template <int LOGX, int LOGY> struct Geo2D {
     static constexpr int DX = 1 << LOGX, DY = 1 << LOGY;
     static constexpr bool PAIRED = LOGY == 7;
-    static constexpr int LX = DX / 16, LY = 16;               // lanes per column / per row-pass group
+    static constexpr bool WIDE = LOGY >= 9;                   // rows of 512 / 1024: 32 / 64 lanes per row
+    static constexpr int LX = DX / 16, LY = WIDE ? DY / 16 : 16;   // lanes per column / per row-pass group
     static constexpr int GY = 1024 / LY;                      // lane groups of the row pass
     static constexpr int RPP = PAIRED ? 2 * GY : GY;          // rows per pass
     static constexpr int ITY = DX / RPP;                      // row passes per image
-    static constexpr int MMY = PAIRED ? 8 : 4;                // modes per lane after one row pass
+    static constexpr int MMY = PAIRED ? 8 : 64 / LY;          // modes per lane after one row pass
     static constexpr int MMX = 64 / LX;                       // modes per lane after the column pass
     static constexpr int COLT = 64 * LX;                      // threads that take part in the column pass
     static constexpr int TILE = DX * TPITCH;
     static constexpr int LDS_MAIN = EXCH_ELEMS > TILE ? EXCH_ELEMS : TILE;   // exchange regions alias the tile
-    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(LDS_MAIN + 2 * kTwLdsSize);
-    static_assert(LOGY == 7 || LOGY == 8, "rows of 128 or 256");
-    static_assert(ITY >= 1 && COLT <= 1024, "unsupported image shape");
+    // after them: first-pass twiddles of the rows (one table row per lane of a group) and of the columns, and for rows
+    // of 512 / 1024 the powers w_LY^e, e < LY, of the second pass
+    static constexpr int TWY_ELEMS = LY * kTwLdsPitch, WSM_ELEMS = WIDE ? LY : 0;
+    static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(LDS_MAIN + TWY_ELEMS + kTwLdsSize + WSM_ELEMS);
+    static_assert(LOGY >= 7 && LOGY <= 10, "rows of 128 to 1024");
+    static_assert(ITY >= 1 && COLT <= 1024 && GY * LY * 17 <= EXCH_ELEMS, "unsupported image shape");
     // element offset of the lane's i-th sample from its first one
     // (logr: the rows of the image lie 2^logr rows of the array apart, see the decimated images below)
     static __device__ __forceinline__ constexpr int sample_off(int i, int logr = 0)
     {
-        return PAIRED ? (i & 7) * 16 + (i >> 3) * ((4 * DY) << logr) : 16 * i;
+        return PAIRED ? (i & 7) * 16 + (i >> 3) * ((4 * DY) << logr) : LY * i;
+    }
+    // column of the redistribution tile (mode along Y) that lane t of a row group holds in slot mm: after the forward
+    // row pass / before the backward one (they differ for rows of 512 / 1024 only)
+    static __device__ __forceinline__ constexpr int col_after_forward(int t, int mm)
+    {
+        return PAIRED ? (t & 7) + 8 * mm : WIDE ? wide_rows_mode<LY>(t, mm) : t + 16 * mm;
+    }
+    static __device__ __forceinline__ constexpr int col_before_backward(int t, int mm)
+    {
+        return PAIRED ? (t & 7) + 8 * mm : t + LY * mm;
     }
 };
 
@@ -57,10 +71,12 @@ template <int LOGX, int LOGY> struct Geo2D {
 //   rows of 256: one row per group; groups 2j, 2j+1 get rows 8 apart.
 //   rows of 128: group g owns rows a and a + 4 (lanes 0-7 / 8-15 finish one each: 16 banks apart), a enumerating the
 //   rows with bit 2 clear; groups 2j, 2j+1 again 8 rows apart.
-template <bool PAIRED> __device__ __forceinline__ int first_row_in_pass(int g)
+//   rows of 512 / 1024: one row per group, a group is at least half a wavefront: any order.
+template <bool PAIRED, bool WIDE = false> __device__ __forceinline__ int first_row_in_pass(int g)
 {
     const int jh = g & 1, rest = g >> 1;
-    if constexpr (!PAIRED) return jh * 8 + (rest % 8) + (rest / 8) * 16;
+    if constexpr (WIDE) return g;
+    else if constexpr (!PAIRED) return jh * 8 + (rest % 8) + (rest / 8) * 16;
     else {
         const int s = jh * 4 + (rest % 4) + (rest / 4) * 8;    // pair index, partner groups 4 apart
         return (s & 3) + 8 * (s >> 2);
@@ -112,19 +128,20 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
     float2* exch_y = lds + gy * (LY * 17);
     float2* exch_x = lds + gx * (LX * 17);
     float2* twtab_y = lds + G::LDS_MAIN;               // after the exchange regions / tile
-    float2* twtab_x = twtab_y + kTwLdsSize;
-    fill_lds_twiddles<LOGY>(twtab_y, tid, 1024);
+    float2* twtab_x = twtab_y + G::TWY_ELEMS;
+    float2* wsm = twtab_x + kTwLdsSize;
+    float2* twsub = wsm + G::WSM_ELEMS;                // decimated images: w^(r p) of the long axis, r < R, p < 64
+    fill_lds_twiddles<LOGY, LY>(twtab_y, tid, 1024);
     fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
+    if (G::WIDE && tid < LY) wsm[tid] = kTwiddle1024[tid * (1024 / LY)];
     const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
-    float2* twsub = twtab_x + kTwLdsSize;              // decimated images: w^(r p) of the long axis, r < R, p < 64
     if constexpr (LOGR > 0) fill_decimation_twiddles<LOGX + LOGR>(twsub, tid, 1024);
     __syncthreads();
 
-    const int row0 = first_row_in_pass<G::PAIRED>(gy);
+    const int row0 = first_row_in_pass<G::PAIRED, G::WIDE>(gy);
     // row the lane finishes after the exchange, and its first mode (paired rows: lanes 8-15 take the second row)
     const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;
-    const int tq = G::PAIRED ? (ty & 7) : ty;
     // scalar base + 32-bit lane offset keeps the load addresses out of the vector registers
     const unsigned lane_off = (unsigned)(((row0 * DY) << LOGR) + ty);
     // x is streamed exactly once: non-temporal loads keep it from evicting the 64x64 spectra, which the
@@ -157,7 +174,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
                 if (it + 1 < ITY) issue(v, img_row, it + 1, lane_off);
                 else issue(v, pre_row, 0, pre_off);
                 fwd_pass1_lds_finish(bb, twrow_y, gg);
-                group_forward_finish<8>(gg, exch_y, ty, T[it]);
+                if constexpr (G::WIDE) wide_rows_forward_finish<LY>(gg, exch_y, wsm, ty, T[it]);
+                else group_forward_finish<8>(gg, exch_y, ty, T[it]);
             } else {
                 cpx gg[16], b8[8];
                 {
@@ -186,7 +204,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
             for (int mm = 0; mm < MMY; ++mm)
-                lds[(trow + G::RPP * it) * TPITCH + tq + (G::PAIRED ? 8 : 16) * mm] = T[it][mm];
+                lds[(trow + G::RPP * it) * TPITCH + G::col_after_forward(ty, mm)] = T[it][mm];
         __syncthreads();
         // pass 2: columns (along X); group gx owns column q = gx, lane tx holds rows tx + LX i
         cpx c[16];
@@ -244,18 +262,19 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     float2* exch_y = lds + gy * (LY * 17);
     float2* exch_x = lds + gx * (LX * 17);
     float2* twtab_y = lds + G::LDS_MAIN;
-    float2* twtab_x = twtab_y + kTwLdsSize;
-    fill_lds_twiddles<LOGY>(twtab_y, tid, 1024);
+    float2* twtab_x = twtab_y + G::TWY_ELEMS;
+    float2* wsm = twtab_x + kTwLdsSize;
+    float2* twsub = wsm + G::WSM_ELEMS;
+    fill_lds_twiddles<LOGY, LY>(twtab_y, tid, 1024);
     fill_lds_twiddles<LOGX>(twtab_x, tid, 1024);
+    if (G::WIDE && tid < LY) wsm[tid] = kTwiddle1024[tid * (1024 / LY)];
     const float2* twrow_y = twtab_y + ty * kTwLdsPitch;
     const float2* twrow_x = twtab_x + tx * kTwLdsPitch;
-    float2* twsub = twtab_x + kTwLdsSize;
     if constexpr (LOGR > 0) fill_decimation_twiddles<LOGX + LOGR>(twsub, tid, 1024);
     __syncthreads();
 
-    const int row0 = first_row_in_pass<G::PAIRED>(gy);
+    const int row0 = first_row_in_pass<G::PAIRED, G::WIDE>(gy);
     const int trow = G::PAIRED ? row0 + 4 * (ty >> 3) : row0;      // row whose modes the lane takes from the tile
-    const int tq = G::PAIRED ? (ty & 7) : ty;
     const unsigned lane_off = (unsigned)(((row0 * DY) << LOGR) + ty);
     const bool col_thread = tid < G::COLT;
     // part r of a decimated image is transformed from the spectrum of the whole image
@@ -323,7 +342,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
             for (int mm = 0; mm < MMY; ++mm)
-                cc[it][mm] = lds[(trow + G::RPP * it) * TPITCH + tq + (G::PAIRED ? 8 : 16) * mm];
+                cc[it][mm] = lds[(trow + G::RPP * it) * TPITCH + G::col_before_backward(ty, mm)];
         __syncthreads();
         // pass 2: rows (q -> y), coalesced row stores.
         // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
@@ -333,6 +352,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
             if (SHARE && (it < it0 || it >= it1)) continue;       // uniform: row passes of the split image left to the partner
             cpx yv[16];
             if constexpr (G::PAIRED) rows128_backward(cc[it], twrow_y, exch_y, ty, yv);
+            else if constexpr (G::WIDE) wide_rows_backward<LY>(cc[it], twrow_y, wsm, exch_y, ty, yv);
             else group_backward_lds<8>(cc[it], twrow_y, exch_y, ty, yv);
             // uniform base + lane offset + immediates
             float2* dst = y + (first_array_row<LOGX, LOGR>(img, nfull) + ((G::RPP * it) << LOGR)) * (long)DY;
@@ -684,18 +704,27 @@ static hipError_t launch_image_kernel(bool inverse, const float2* in, float2* ou
     return hipGetLastError();
 }
 
-// DX of 512 or 1024: two or four decimated parts of 256 rows each
 static hipError_t dispatch_image_kernel(bool inverse, int logDX, int logDY, const float2* in, float2* out, int nimg,
                                         hipStream_t stream)
 {
-    if (logDX == 8 && logDY == 8) return launch_image_kernel<8, 8, 0>(inverse, in, out, nimg, stream);
-    if (logDX == 8 && logDY == 7) return launch_image_kernel<8, 7, 0>(inverse, in, out, nimg, stream);
-    if (logDX == 7 && logDY == 8) return launch_image_kernel<7, 8, 0>(inverse, in, out, nimg, stream);
-    if (logDX == 7 && logDY == 7) return launch_image_kernel<7, 7, 0>(inverse, in, out, nimg, stream);
-    if (logDX == 9 && logDY == 8) return launch_image_kernel<8, 8, 1>(inverse, in, out, nimg, stream);
-    if (logDX == 9 && logDY == 7) return launch_image_kernel<8, 7, 1>(inverse, in, out, nimg, stream);
-    if (logDX == 10 && logDY == 8) return launch_image_kernel<8, 8, 2>(inverse, in, out, nimg, stream);
-    if (logDX == 10 && logDY == 7) return launch_image_kernel<8, 7, 2>(inverse, in, out, nimg, stream);
+    // columns: 128 or 256 rows per block, 512 / 1024 as 2 / 4 parts of 256; rows: any built length
+    auto with_rows = [&](auto logy) -> hipError_t {
+        constexpr int LOGY = decltype(logy)::value;
+        switch (logDX) {
+        case 7: return launch_image_kernel<7, LOGY, 0>(inverse, in, out, nimg, stream);
+        case 8: return launch_image_kernel<8, LOGY, 0>(inverse, in, out, nimg, stream);
+        case 9: return launch_image_kernel<8, LOGY, 1>(inverse, in, out, nimg, stream);
+        case 10: return launch_image_kernel<8, LOGY, 2>(inverse, in, out, nimg, stream);
+        default: return hipErrorInvalidValue;
+        }
+    };
+    switch (logDY) {
+    case 7: return with_rows(std::integral_constant<int, 7>{});
+    case 8: return with_rows(std::integral_constant<int, 8>{});
+    case 9: return with_rows(std::integral_constant<int, 9>{});
+    case 10: return with_rows(std::integral_constant<int, 10>{});
+    default: break;
+    }
     return hipErrorInvalidValue;
 }
 
