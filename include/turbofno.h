@@ -87,8 +87,8 @@ int turbofno_layer_1d(int bs, int dimX, int DY, int K, int N, const void* x, con
  * intermediates t1/t2 in buffers owned by main(); here the caller passes `workspace` of at least
  * turbofno_layer_2d_workspace_bytes(...) bytes (256-byte aligned). x is not modified.
  * algo: TURBOFNO_2D_AUTO picks by size (lengths up to 256: WHOLE_IMAGE from a batch of 8, and from a batch of 4 when
- * there are enough images; THREE_KERNEL below; longer axes: WHOLE_IMAGE from several hundred MiB of input and output,
- * for rows of 1024 from several GiB, else ROWS_FIRST or THREE_KERNEL); the workspace query with the same arguments,
+ * there are enough images; THREE_KERNEL below; longer axes: WHOLE_IMAGE from 0.6 to 4.5 GiB of input and output,
+ * depending on the lengths, else ROWS_FIRST or THREE_KERNEL); the workspace query with the same arguments,
  * and turbofno_query_2d_algo, make the same
  * choice. Every algorithm takes every pair of lengths in {128, 256, 512, 1024} (WHOLE_IMAGE handles images of 512 or
  * 1024 rows as two or four interleaved parts of 256 rows that the contraction sums over). ROWS_FIRST is the three-stage structure with the axes exchanged

@@ -52,21 +52,24 @@ def test_large_grids_and_long_axes():
     assert tf.query_2d_algo(2, 512, 512, 64, 64) == tf.ALGO_ROWS_FIRST
     assert tf.query_2d_algo(1, 512, 512, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(8, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
-    assert tf.query_2d_algo(8, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(4, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(2, 1024, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
-    # large ones: the whole-image kernels (512 / 1024 rows as interleaved parts of 256, long rows with 32 / 64 lanes)
+    # large ones: the whole-image kernels (512 / 1024 rows as interleaved parts of 256, long rows with 32 / 64 lanes),
+    # from a volume of input and output that depends on the lengths
     assert tf.query_2d_algo(16, 512, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(4, 512, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE            # 768 MiB
     assert tf.query_2d_algo(4, 512, 512, 16, 64) == tf.ALGO_THREE_KERNEL           # 640 MiB
     assert tf.query_2d_algo(16, 512, 256, 32, 64) == tf.ALGO_WHOLE_IMAGE
-    assert tf.query_2d_algo(4, 512, 256, 32, 64) == tf.ALGO_THREE_KERNEL
+    assert tf.query_2d_algo(4, 512, 256, 32, 64) == tf.ALGO_THREE_KERNEL           # 384 MiB
     assert tf.query_2d_algo(16, 512, 128, 32, 64) == tf.ALGO_WHOLE_IMAGE
     assert tf.query_2d_algo(8, 512, 128, 32, 64) == tf.ALGO_THREE_KERNEL
     assert tf.query_2d_algo(16, 256, 512, 32, 64) == tf.ALGO_WHOLE_IMAGE
-    assert tf.query_2d_algo(32, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL
-    assert tf.query_2d_algo(16, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST
-    assert tf.query_2d_algo(16, 256, 1024, 32, 128) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(8, 1024, 256, 32, 64) == tf.ALGO_WHOLE_IMAGE           # 1536 MiB
+    assert tf.query_2d_algo(4, 1024, 256, 32, 64) == tf.ALGO_THREE_KERNEL          # 768 MiB
+    assert tf.query_2d_algo(16, 256, 1024, 32, 64) == tf.ALGO_WHOLE_IMAGE          # 3072 MiB
+    assert tf.query_2d_algo(8, 256, 1024, 32, 64) == tf.ALGO_ROWS_FIRST            # 1536 MiB
     assert tf.query_2d_algo(16, 1024, 1024, 32, 64) == tf.ALGO_WHOLE_IMAGE
+    assert tf.query_2d_algo(4, 1024, 1024, 32, 64) == tf.ALGO_ROWS_FIRST           # 3072 MiB
 
 
 def test_queries_answer_zero_for_arguments_the_calls_refuse():

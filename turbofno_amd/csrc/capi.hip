@@ -62,17 +62,15 @@ int pick_algo(int bs, int DX, int DY, int K, int N, int algo)
     if (DX > 256 || DY > 256) {
         // Long axes on the whole-image kernels (512 / 1024 rows as interleaved parts of 256, rows of 512 / 1024 with 32 /
         // 64 lanes each): x and y move once and nothing but 64 x 64 modes in between, against intermediates of 1/8 (length
-        // 512) or 1/16 (1024) of the data, twice over, for three stages. Measured on MI355X (324 shapes, bs 1-32, all three
-        // paths back to back), with `mib` the input and output in MiB: DX = 512 with rows up to 256 ahead by 3-24 % from
-        // 640 MiB, rows of 512 by 1-22 % from 768 MiB (3 GiB of 512 x 512: 752 -> 608 us); rows of 1024 level with whole
-        // rows first (within 5 %) except for the large problems below (8-16 %); behind by up to 2x on small problems.
+        // 512) or 1/16 (1024) of the data, twice over, for three stages; but one block per part of an image needs enough
+        // of them. Measured on MI355X (348 shapes, bs 1-32, all three paths back to back): ahead from the volume of
+        // input and output below, by 3-10 % there and by 13-34 % at several GiB (3 GiB of 512 x 512: 752 -> 600 us);
+        // behind by up to 2x on small problems.
+        static const int whole_from_mib[4][4] = {       // [log2 DX - 7][log2 DY - 7]
+            { 0, 0, 576, 4608 }, { 0, 0, 768, 3072 }, { 576, 576, 768, 2560 }, { 1152, 1280, 2560, 4608 } };
         const long mib = ((long)K + N) * bs * DX * DY >> 17;
-        bool whole;
-        if (DY <= 256) whole = DX == 512 && mib >= 640;
-        else if (DY == 512) whole = mib >= 768;
-        else whole = (DX == 256 && N >= 128 && mib >= 4608) || (DX == 512 && mib >= 4608 && (N >= 128 || bs >= 16)) ||
-                     (DX == 1024 && mib >= 9216);
-        if (whole) return TURBOFNO_2D_WHOLE_IMAGE;
+        const int lx = log2_exact(DX) - 7, ly = log2_exact(DY) - 7;
+        if (lx >= 0 && lx < 4 && ly >= 0 && ly < 4 && mib >= whole_from_mib[lx][ly]) return TURBOFNO_2D_WHOLE_IMAGE;
     }
     if (DX > 256 || DY > 256) {
         // otherwise three stages. The axis that is transformed first is the one whose

@@ -189,56 +189,74 @@ TFNO_DEV void rows128_backward(const cpx (&c)[8], const TW& twrow, cpx* exch, in
 }
 
 // Rows of 512 / 1024 in the whole-image kernels: a group of L = 32 / 64 lanes owns one row, lane t holds samples t + L i.
-// The scheme of the wide_* codelets, with every twiddle taken from LDS (a global load inside the row loop would queue
-// behind the loads of the next row, which are in flight all the time): twrow = the lane's row of the first-pass table,
-// wsm[e] = w_L^e, e < L.
-// g[]: first-pass results, already twiddled. Lane t = A r + a (A = L / 16) finishes the modes r + 16 (a + A j), j < 64 / L,
-// in out[j]: for one j the lanes of a group hold L consecutive modes, so that they can be written to one row of a tile
-// without bank conflicts (the map of the 1D kernels, wide_mode, puts lanes 32 modes apart).
-template <int L> TFNO_DEV constexpr int wide_rows_mode(int t, int j) { return t / (L / 16) + 16 * (t % (L / 16) + (L / 16) * j); }
+// The scheme of the wide_* codelets (inner 16-point transforms over the lanes tt = a + A b, A = L / 16, then a sum over
+// a), with every twiddle taken from LDS (a global load inside the row loop would queue behind the loads of the next row,
+// which are in flight all the time): twrow = the lane's row of the first-pass table, wsm[e] = w_L^e, e < L. The lanes
+// and the two exchanges are laid out for the LDS banks (64 banks of 4 bytes, 32 lanes of 8 bytes per cycle):
+//   second-pass lane t = 16 a + r computes inner_a[c] of bin r, then finishes the modes r + 16 (a + A j) = t + L j: the
+//     natural order, L consecutive modes per slot j;
+//   first exchange: the A rows a + A b of one b side by side, [b][a][16 bins] with a pitch of 16 A + 1: the read of one b
+//     covers 32 consecutive elements per half wavefront, the write of one bin is conflict-free for L = 32 (2-way for 64);
+//   second exchange: [c][16 a' + r] with a pitch of L + 16: writes are consecutive, and the lanes a and a + 1 of a half
+//     wavefront, which read the rows c = a + A j and c + 1, land 16 elements apart modulo 32.
+// g[]: first-pass results, already twiddled. On return out[j] = mode t + L j.
 template <int L>
 TFNO_DEV void wide_rows_forward_finish(const cpx (&g)[16], cpx* exch, const cpx* wsm, int t, cpx (&out)[64 / L])
 {
-    constexpr int A = L / 16, MM = 64 / L;
-    const int r = t / A, a = t % A;
+    constexpr int A = L / 16, MM = 64 / L, P1 = 16 * A + 1, PS = L + 16;
+    static_assert(16 * P1 <= L * 17 && 4 * PS <= L * 17, "both exchanges fit the group's region");
+    const int r = t % 16, a = t / 16;
     wave_lds_fence();
 #pragma unroll
-    for (int k = 0; k < 16; ++k) exch[t * 17 + k] = g[k];
+    for (int k = 0; k < 16; ++k) exch[(t / A) * P1 + (t % A) * 16 + k] = g[k];
     wave_lds_fence();
     cpx inner[4];
-    wide_forward_inner<L>(exch, 1, t, inner);
+    {
+        cpx u[16];
+#pragma unroll
+        for (int b = 0; b < 16; ++b) u[b] = exch[b * P1 + t];      // lane tt = a + A b, bin r
+        dft16_first4<-1>(u, inner);
+    }
     wave_lds_fence();                                // every lane of the group has read the first exchange
 #pragma unroll
-    for (int c = 0; c < 4; ++c) exch[wide_swap_index<L>(r, c, a)] = inner[c];
+    for (int c = 0; c < 4; ++c) exch[c * PS + t] = inner[c];
     wave_lds_fence();
 #pragma unroll
     for (int j = 0; j < MM; ++j) {
         const int c = a + A * j;
-        cpx acc = exch[wide_swap_index<L>(r, c, 0)];
+        cpx acc = exch[c * PS + r];
 #pragma unroll
-        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[wide_swap_index<L>(r, c, ap)], wsm[(ap * c) % L]);
+        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[c * PS + 16 * ap + r], wsm[(ap * c) % L]);
         out[j] = acc;
     }
 }
 
 // c[mm] = mode t + L mm of the row. On return y[i] = sample t + L i.
+// Lane l = (t1 = l % Q, rq = l / Q), Q = L / 4, forms the first-pass inputs of the four lanes t1 + Q t2 for the bins
+// r = rq + 4 ri (wide_backward_partial_tw) and parks them for their owners at [r][lane ^ (Q rq)], rows of L: the owners
+// read a row as L consecutive elements, and the XOR puts the four rq of one write Q elements apart, so that the 32
+// lanes of a half wavefront hit 32 different bank pairs in both directions.
 template <int L>
 TFNO_DEV void wide_rows_backward(const cpx (&c)[64 / L], const cpx* twrow, const cpx* wsm, cpx* exch, int t, cpx (&y)[16])
 {
+    constexpr int Q = L / 4;
+    static_assert(16 * L <= L * 17, "the parked values fit the group's region");
     wave_lds_fence();
 #pragma unroll
     for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
     wave_lds_fence();
     cpx part[16];
-    const int t1 = t % (L / 4);
+    const int t1 = t % Q, rq = t / Q;
     wide_backward_partial_tw<L>(exch, 1, t, wsm[t1], wsm[2 * t1], wsm[3 * t1], part);
     wave_lds_fence();                                // every lane of the group has read the 64 modes
 #pragma unroll
-    for (int k = 0; k < 16; ++k) exch[wide_back_index<L>(t, k)] = part[k];
+    for (int ri = 0; ri < 4; ++ri)
+#pragma unroll
+        for (int t2 = 0; t2 < 4; ++t2) exch[(rq + 4 * ri) * L + t1 + Q * (t2 ^ rq)] = part[4 * ri + t2];
     wave_lds_fence();
     cpx e[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+    for (int r = 0; r < 16; ++r) e[r] = exch[r * L + (t ^ (Q * (r & 3)))];
     inv_pass2_lds(e, twrow, y);
 }
 

@@ -54,16 +54,8 @@ template <int LOGX, int LOGY> struct Geo2D {
     {
         return PAIRED ? (i & 7) * 16 + (i >> 3) * ((4 * DY) << logr) : LY * i;
     }
-    // column of the redistribution tile (mode along Y) that lane t of a row group holds in slot mm: after the forward
-    // row pass / before the backward one (they differ for rows of 512 / 1024 only)
-    static __device__ __forceinline__ constexpr int col_after_forward(int t, int mm)
-    {
-        return PAIRED ? (t & 7) + 8 * mm : WIDE ? wide_rows_mode<LY>(t, mm) : t + 16 * mm;
-    }
-    static __device__ __forceinline__ constexpr int col_before_backward(int t, int mm)
-    {
-        return PAIRED ? (t & 7) + 8 * mm : t + LY * mm;
-    }
+    // column of the redistribution tile (mode along Y) that lane t of a row group holds in slot mm
+    static __device__ __forceinline__ constexpr int tile_col(int t, int mm) { return PAIRED ? (t & 7) + 8 * mm : t + LY * mm; }
 };
 
 // First row (within one pass) of lane group g. The two groups that share an LDS cycle (one half wavefront) must
@@ -88,16 +80,34 @@ template <bool PAIRED, bool WIDE = false> __device__ __forceinline__ int first_r
 //     X[p] = sum_{r<R} w_{R DX}^(r p) * DFT_DX(part r)[p],    p < 64
 // so the forward kernel transforms every part like an image of its own and multiplies its 64 x 64 modes by w^(r p); the
 // sum over r is a sum over "channels" and is done by the contraction that follows (channel r K + k, weight W[k]): the
-// parts are numbered r * nfull + image for that, nfull whole images. Backward, the R parts of an output image are
-// transformed from the one spectrum of the image, multiplied by conj(w^(r p)). Nothing but x, y and the 64 x 64 modes
-// ever leaves a CU, as for images of one block.
-template <int LOGX, int LOGR> __device__ __forceinline__ long first_array_row(long img, int nfull)
-{
-    if constexpr (LOGR == 0) return img << LOGX;
-    else {
-        const unsigned part = (unsigned)img / (unsigned)nfull, image = (unsigned)img - part * (unsigned)nfull;
-        return ((long)image << (LOGX + LOGR)) + part;
+// spectrum of part r of image i is stored at index r * nfull + i for that, nfull whole images. Backward, the R parts of
+// an output image are transformed from the one spectrum of the image, multiplied by conj(w^(r p)). Nothing but x, y and
+// the 64 x 64 modes ever leaves a CU, as for images of one block.
+//
+// Numbering of the block-images (one per block iteration). Side by side: image * R + part, the parts of an image run on
+// neighbouring blocks at the same time and all rows of the array are in flight together, not every R-th one; part major:
+// part * nfull + image. Measured: the forward kernels are 2-9 % faster side by side everywhere; the backward kernels as
+// well for four parts and for rows up to 256, but 3 % slower for two parts of rows of 512 / 1024, which keep part major.
+template <int LOGR, bool PART_MAJOR> struct PartNumbering {
+    static constexpr int R = 1 << LOGR;
+    static __device__ __forceinline__ unsigned part(long img, int nfull)
+    {
+        if constexpr (LOGR == 0) return 0;
+        else if constexpr (PART_MAJOR) return (unsigned)img / (unsigned)nfull;
+        else return (unsigned)img & (R - 1);
     }
+    static __device__ __forceinline__ long image(long img, int nfull)
+    {
+        if constexpr (LOGR == 0) return img;
+        else if constexpr (PART_MAJOR) return (unsigned)img % (unsigned)nfull;
+        else return img >> LOGR;
+    }
+};
+// first row in the array of block-image img: row `part` of image `image`, whose rows lie R rows apart
+template <int LOGX, int LOGR, bool PART_MAJOR> __device__ __forceinline__ long first_array_row(long img, int nfull)
+{
+    using P = PartNumbering<LOGR, PART_MAJOR>;
+    return (P::image(img, nfull) << (LOGX + LOGR)) + P::part(img, nfull);
 }
 constexpr int kDecimationTwiddles = 64 * 4;      // complex elements: R <= 4 parts
 template <int LOGD> __device__ __forceinline__ void fill_decimation_twiddles(float2* tab, int tid, int nthreads)
@@ -153,14 +163,14 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
     };
 
     long img = blockIdx.x;
-    long img_row = first_array_row<LOGX, LOGR>(img < nimg ? img : 0, nfull);
+    long img_row = first_array_row<LOGX, LOGR, false>(img < nimg ? img : 0, nfull);
     cpx v[16];
     if (img < nimg) issue(v, img_row, 0, lane_off);
     for (; img < nimg; img += gridDim.x) {
         // look-ahead target: the next image's first rows; after the last image every lane group re-reads the
         // same row (row 0 of image 0, cache resident) so the loop stays branch free at no HBM cost
         const bool more = img + gridDim.x < nimg;
-        const long pre_row = first_array_row<LOGX, LOGR>(more ? img + gridDim.x : 0, nfull);
+        const long pre_row = first_array_row<LOGX, LOGR, false>(more ? img + gridDim.x : 0, nfull);
         const unsigned pre_off = more ? lane_off : (unsigned)ty;
         // pass 1: rows (along Y). T[it][mm] = mode tq + 16 mm (paired rows: tq + 8 mm) of row trow + RPP it
         cpx T[ITY][MMY];
@@ -204,7 +214,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
             for (int mm = 0; mm < MMY; ++mm)
-                lds[(trow + G::RPP * it) * TPITCH + G::col_after_forward(ty, mm)] = T[it][mm];
+                lds[(trow + G::RPP * it) * TPITCH + G::tile_col(ty, mm)] = T[it][mm];
         __syncthreads();
         // pass 2: columns (along X); group gx owns column q = gx, lane tx holds rows tx + LX i
         cpx c[16];
@@ -219,7 +229,7 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
             group_forward_finish<LOGX>(gg, exch_x, tx, z);
             if constexpr (LOGR > 0) {
                 // part r of a decimated image: its modes enter the sum over the parts with w^(r p) of the long axis
-                const unsigned r = (unsigned)img / (unsigned)nfull;
+                const int r = (int)PartNumbering<LOGR, false>::part(img, nfull);
                 if (r != 0) {
 #pragma unroll
                     for (int mm = 0; mm < MMX; ++mm) z[mm] = cmul(z[mm], twsub[r * 64 + tx + LX * mm]);
@@ -227,7 +237,8 @@ __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restr
             }
             // lane order of the retained modes: element mm*COLT + q*LX + tx  <->  mode (p = tx + LX mm, q).
             // Written through as it is produced, so the end-of-kernel cache write-back has nothing left to flush
-            float2* dst = spec + img * 4096;
+            // (decimated images: the spectrum of part r of image i is channel r of the contraction, index r * nfull + i)
+            float2* dst = spec + (PartNumbering<LOGR, false>::part(img, nfull) * (long)nfull + PartNumbering<LOGR, false>::image(img, nfull)) * 4096;
 #pragma unroll
             for (int mm = 0; mm < MMX; ++mm) store_streaming(dst + tid + G::COLT * mm, z[mm]);
         }
@@ -278,7 +289,9 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
     const unsigned lane_off = (unsigned)(((row0 * DY) << LOGR) + ty);
     const bool col_thread = tid < G::COLT;
     // part r of a decimated image is transformed from the spectrum of the whole image
-    auto spectrum_of = [&](long img) { return spec + (LOGR > 0 ? (long)((unsigned)img % (unsigned)nfull) : img) * 4096; };
+    constexpr bool PART_MAJOR = LOGR == 1 && LOGY >= 9;
+    using Parts = PartNumbering<LOGR, PART_MAJOR>;
+    auto spectrum_of = [&](long img) { return spec + Parts::image(img, nfull) * 4096; };
 
     // The block transforms `count` images, image_at(k) for k < count; of its last one, if `split`, only the row passes
     // [pass0, pass1). Without SHARE: every block the images blockIdx.x, + gridDim.x, ... in full.
@@ -319,7 +332,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
         // pass 1: columns (p -> x) of column q = gx
         cpx u[16];
         if constexpr (LOGR > 0) {
-            const unsigned r = (unsigned)img / (unsigned)nfull;
+            const int r = (int)Parts::part(img, nfull);
             if (r != 0 && col_thread) {
 #pragma unroll
                 for (int mm = 0; mm < MMX; ++mm) c[mm] = cmulc(c[mm], twsub[r * 64 + tx + LX * mm]);
@@ -342,7 +355,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
         for (int it = 0; it < ITY; ++it)
 #pragma unroll
             for (int mm = 0; mm < MMY; ++mm)
-                cc[it][mm] = lds[(trow + G::RPP * it) * TPITCH + G::col_before_backward(ty, mm)];
+                cc[it][mm] = lds[(trow + G::RPP * it) * TPITCH + G::tile_col(ty, mm)];
         __syncthreads();
         // pass 2: rows (q -> y), coalesced row stores.
         // y is written once and not re-read by this layer: non-temporal stores stop half a gigabyte of
@@ -355,7 +368,7 @@ __global__ __launch_bounds__(1024) void ifft2d_pad_kernel(const float2* __restri
             else if constexpr (G::WIDE) wide_rows_backward<LY>(cc[it], twrow_y, wsm, exch_y, ty, yv);
             else group_backward_lds<8>(cc[it], twrow_y, exch_y, ty, yv);
             // uniform base + lane offset + immediates
-            float2* dst = y + (first_array_row<LOGX, LOGR>(img, nfull) + ((G::RPP * it) << LOGR)) * (long)DY;
+            float2* dst = y + (first_array_row<LOGX, LOGR, PART_MAJOR>(img, nfull) + ((G::RPP * it) << LOGR)) * (long)DY;
 #pragma unroll
             for (int i = 0; i < 16; ++i) store_streaming(dst + lane_off + G::sample_off(i, LOGR), yv[i]);
         }
