@@ -1,5 +1,5 @@
 // Transforms of one signal by one L-lane group of a wavefront (L = D/16 lanes, 16 samples per lane; L = 8, 16 for
-// lengths 128, 256 and, with direct second-pass sums, L = 32, 64 for lengths 512, 1024), built from the register
+// lengths 128, 256 and, with a pruned second pass in two steps, L = 32, 64 for lengths 512, 1024), built from the register
 // codelets plus one padded LDS exchange that stays inside the wavefront (no block barrier). Shared by the fused 1D kernel and the 2D image kernels.
 #pragma once
 #include "fft_codelets.h"
@@ -19,21 +19,99 @@ template <int LOGDY> struct Geo1D {
     static constexpr size_t LDS_BYTES = sizeof(float2) * (size_t)(GROUPS * SA_PITCH + GROUPS * SW_PITCH + GROUPS * EXCH);
 };
 
+// Lengths 512 / 1024: a group of L = 32 / 64 lanes owns one signal, lane t holds samples t + L i. The scheme of the wide_*
+// codelets (inner 16-point transforms over the lanes tt = a + A b, A = L / 16, then a sum over a), with the lanes and the
+// two exchanges laid out for the LDS banks (64 banks of 4 bytes, 32 lanes of 8 bytes per cycle):
+//   second-pass lane t = 16 a + r computes inner_a[c] of bin r, then finishes the modes r + 16 (a + A j) = t + L j: the
+//     natural order, L consecutive modes per slot j;
+//   first exchange: the A rows a + A b of one b side by side, [b][a][16 bins] with a pitch of 16 A + 1: the read of one b
+//     covers 32 consecutive elements per half wavefront, the write of one bin is conflict-free for L = 32 (2-way for 64);
+//   second exchange: [c][16 a' + r] with a pitch of L + 16: writes are consecutive, and the lanes a and a + 1 of a half
+//     wavefront, which read the rows c = a + A j and c + 1, land 16 elements apart modulo 32.
+// wpow(e) = w_L^e, e < L: from the constant table, or from LDS where a global load would be in the way.
+// g[]: first-pass results, already twiddled. On return out[j] = mode t + L j.
+template <int L, class Pow>
+TFNO_DEV void wide_forward_finish(const cpx (&g)[16], cpx* exch, Pow wpow, int t, cpx (&out)[64 / L])
+{
+    constexpr int A = L / 16, MM = 64 / L, P1 = 16 * A + 1, PS = L + 16;
+    static_assert(16 * P1 <= L * 17 && 4 * PS <= L * 17, "both exchanges fit the group's region");
+    const int r = t % 16, a = t / 16;
+    wave_lds_fence();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) exch[(t / A) * P1 + (t % A) * 16 + k] = g[k];
+    wave_lds_fence();
+    cpx inner[4];
+    {
+        cpx u[16];
+#pragma unroll
+        for (int b = 0; b < 16; ++b) u[b] = exch[b * P1 + t];      // lane tt = a + A b, bin r
+        dft16_first4<-1>(u, inner);
+    }
+    wave_lds_fence();                                // every lane of the group has read the first exchange
+#pragma unroll
+    for (int c = 0; c < 4; ++c) exch[c * PS + t] = inner[c];
+    wave_lds_fence();
+#pragma unroll
+    for (int j = 0; j < MM; ++j) {
+        const int c = a + A * j;
+        cpx acc = exch[c * PS + r];
+#pragma unroll
+        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[c * PS + 16 * ap + r], wpow((ap * c) % L));
+        out[j] = acc;
+    }
+}
+
+// Backward, up to the inputs of the last pass: c[mm] = mode t + L mm; on return e[r] = first-pass input r of lane t
+// (before the conjugate twiddle). Lane l = (t1 = l % Q, rq = l / Q), Q = L / 4, forms the inputs of the four lanes
+// t1 + Q t2 for the bins r = rq + 4 ri (wide_backward_partial_tw) and parks them for their owners at
+// [r][lane ^ (Q rq)], rows of L: the owners read a row as L consecutive elements, and the XOR puts the four rq of one
+// write Q elements apart, so that the 32 lanes of a half wavefront hit 32 different bank pairs in both directions.
+template <int L, class Pow>
+TFNO_DEV void wide_backward_inputs(const cpx (&c)[64 / L], Pow wpow, cpx* exch, int t, cpx (&e)[16])
+{
+    constexpr int Q = L / 4;
+    wave_lds_fence();
+#pragma unroll
+    for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
+    wave_lds_fence();
+    cpx part[16];
+    const int t1 = t % Q, rq = t / Q;
+    wide_backward_partial_tw<L>(exch, 1, t, wpow(t1), wpow(2 * t1), wpow(3 * t1), part);
+    wave_lds_fence();                                // every lane of the group has read the 64 modes
+#pragma unroll
+    for (int ri = 0; ri < 4; ++ri)
+#pragma unroll
+        for (int t2 = 0; t2 < 4; ++t2) exch[(rq + 4 * ri) * L + t1 + Q * (t2 ^ rq)] = part[4 * ri + t2];
+    wave_lds_fence();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = exch[r * L + (t ^ (Q * (r & 3)))];
+}
+template <int L> struct TablePow {                   // w_L^e from the constant table
+    TFNO_DEV cpx operator()(int e) const { return kTwiddle1024[(e * (1024 / L)) & 1023]; }
+};
+struct LdsPow {                                      // from an LDS array of the L powers
+    const cpx* w;
+    TFNO_DEV cpx operator()(int e) const { return w[e]; }
+};
+
 // Mode that lane t of an L-lane group holds in out[mm] after a forward transform.
 template <int LOGDY> TFNO_DEV constexpr int forward_mode_of_lane(int t, int mm)
 {
     constexpr int L = (1 << LOGDY) / 16;
-    if constexpr (L >= 32) return wide_mode<L>(t, mm);
-    else return t + L * mm;
+    return t + L * mm;
 }
 
 // second half of the forward transform: exchange of the twiddled first-pass results g[] inside the
-// L-lane group, then the pruned L-point DFT. On return lane `t` holds mode forward_mode_of_lane<LOGDY>(t, mm) in
-// out[mm]: t + L*mm for lengths 128 and 256.
+// L-lane group, then the pruned L-point DFT. On return lane `t` holds mode forward_mode_of_lane<LOGDY>(t, mm) =
+// t + L*mm in out[mm].
 template <int LOGDY>
 TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&out)[Geo1D<LOGDY>::MM])
 {
     constexpr int L = Geo1D<LOGDY>::L;
+    if constexpr (L >= 32) {
+        wide_forward_finish<L>(g, exch, TablePow<L>{}, t, out);
+        return;
+    }
     wave_lds_fence();
 #pragma unroll
     for (int r = 0; r < 16; ++r) exch[t * 17 + r] = g[r];
@@ -43,17 +121,7 @@ TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&o
 #pragma unroll
         for (int tt = 0; tt < 16; ++tt) u[tt] = exch[tt * 17 + t];
         dft16_first4<-1>(u, out);                       // out[s] = X[t + 16 s]
-    } else if constexpr (L >= 32) {
-        // lengths 512 / 1024: pruned second pass with a second small exchange; NOTE the lane-to-mode map of the result
-        // is wide_mode<L>(t, mm), not t + L*mm (forward_mode_of_lane below)
-        cpx inner[4];
-        wide_forward_inner<L>(exch, 1, t, inner);
-        wave_lds_fence();                                // every lane of the group has read the first exchange
-#pragma unroll
-        for (int c = 0; c < 4; ++c) exch[wide_swap_index<L>(t / (L / 16), c, t % (L / 16))] = inner[c];
-        wave_lds_fence();
-        wide_forward_outer<L>(exch, 1, t, out);
-    } else {
+    } else if constexpr (L == 8) {
         cpx u0[8], u1[8], o0[4], o1[4];
 #pragma unroll
         for (int tt = 0; tt < 8; ++tt) { u0[tt] = exch[tt * 17 + t]; u1[tt] = exch[tt * 17 + t + 8]; }
@@ -79,36 +147,26 @@ template <int LOGDY>
 TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[16], cpx* exch, int t, cpx (&y)[16])
 {
     constexpr int L = Geo1D<LOGDY>::L;
-    wave_lds_fence();
-    if constexpr (L >= 32) {
-#pragma unroll
-        for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
-    } else if constexpr (L == 16) {
-        cpx h[16];
-        dft16_pad4<+1>(c, h);
-#pragma unroll
-        for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
-    } else {
-        cpx c0[4], c1[4], h0[8], h1[8];
-#pragma unroll
-        for (int s = 0; s < 4; ++s) { c0[s] = c[2 * s]; c1[s] = c[2 * s + 1]; }
-        dft8_pad4<+1>(c0, h0);
-        dft8_pad4<+1>(c1, h1);
-#pragma unroll
-        for (int tt = 0; tt < 8; ++tt) { exch[tt * 17 + t] = h0[tt]; exch[tt * 17 + t + 8] = h1[tt]; }
-    }
-    wave_lds_fence();
     cpx e[16];
     if constexpr (L >= 32) {
-        cpx part[16];
-        wide_backward_partial<L>(exch, 1, t, part);
-        wave_lds_fence();                               // every lane of the group has read the 64 modes
-#pragma unroll
-        for (int k = 0; k < 16; ++k) exch[wide_back_index<L>(t, k)] = part[k];
-        wave_lds_fence();
-#pragma unroll
-        for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
+        wide_backward_inputs<L>(c, TablePow<L>{}, exch, t, e);
     } else {
+        wave_lds_fence();
+        if constexpr (L == 16) {
+            cpx h[16];
+            dft16_pad4<+1>(c, h);
+#pragma unroll
+            for (int tt = 0; tt < 16; ++tt) exch[tt * 17 + t] = h[tt];
+        } else {
+            cpx c0[4], c1[4], h0[8], h1[8];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) { c0[s] = c[2 * s]; c1[s] = c[2 * s + 1]; }
+            dft8_pad4<+1>(c0, h0);
+            dft8_pad4<+1>(c1, h1);
+#pragma unroll
+            for (int tt = 0; tt < 8; ++tt) { exch[tt * 17 + t] = h0[tt]; exch[tt * 17 + t + 8] = h1[tt]; }
+        }
+        wave_lds_fence();
 #pragma unroll
         for (int r = 0; r < 16; ++r) e[r] = exch[t * 17 + r];
     }
@@ -188,75 +246,20 @@ TFNO_DEV void rows128_backward(const cpx (&c)[8], const TW& twrow, cpx* exch, in
     for (int i = 0; i < 8; ++i) { y[i] = a[i]; y[8 + i] = b[i]; }
 }
 
-// Rows of 512 / 1024 in the whole-image kernels: a group of L = 32 / 64 lanes owns one row, lane t holds samples t + L i.
-// The scheme of the wide_* codelets (inner 16-point transforms over the lanes tt = a + A b, A = L / 16, then a sum over
-// a), with every twiddle taken from LDS (a global load inside the row loop would queue behind the loads of the next row,
-// which are in flight all the time): twrow = the lane's row of the first-pass table, wsm[e] = w_L^e, e < L. The lanes
-// and the two exchanges are laid out for the LDS banks (64 banks of 4 bytes, 32 lanes of 8 bytes per cycle):
-//   second-pass lane t = 16 a + r computes inner_a[c] of bin r, then finishes the modes r + 16 (a + A j) = t + L j: the
-//     natural order, L consecutive modes per slot j;
-//   first exchange: the A rows a + A b of one b side by side, [b][a][16 bins] with a pitch of 16 A + 1: the read of one b
-//     covers 32 consecutive elements per half wavefront, the write of one bin is conflict-free for L = 32 (2-way for 64);
-//   second exchange: [c][16 a' + r] with a pitch of L + 16: writes are consecutive, and the lanes a and a + 1 of a half
-//     wavefront, which read the rows c = a + A j and c + 1, land 16 elements apart modulo 32.
-// g[]: first-pass results, already twiddled. On return out[j] = mode t + L j.
+// Rows of 512 / 1024 in the whole-image kernels: wide_forward_finish / wide_backward_inputs with every twiddle taken
+// from LDS (a global load inside the row loop would queue behind the loads of the next row, which are in flight all
+// the time): twrow = the lane's row of the first-pass table, wsm[e] = w_L^e, e < L.
 template <int L>
 TFNO_DEV void wide_rows_forward_finish(const cpx (&g)[16], cpx* exch, const cpx* wsm, int t, cpx (&out)[64 / L])
 {
-    constexpr int A = L / 16, MM = 64 / L, P1 = 16 * A + 1, PS = L + 16;
-    static_assert(16 * P1 <= L * 17 && 4 * PS <= L * 17, "both exchanges fit the group's region");
-    const int r = t % 16, a = t / 16;
-    wave_lds_fence();
-#pragma unroll
-    for (int k = 0; k < 16; ++k) exch[(t / A) * P1 + (t % A) * 16 + k] = g[k];
-    wave_lds_fence();
-    cpx inner[4];
-    {
-        cpx u[16];
-#pragma unroll
-        for (int b = 0; b < 16; ++b) u[b] = exch[b * P1 + t];      // lane tt = a + A b, bin r
-        dft16_first4<-1>(u, inner);
-    }
-    wave_lds_fence();                                // every lane of the group has read the first exchange
-#pragma unroll
-    for (int c = 0; c < 4; ++c) exch[c * PS + t] = inner[c];
-    wave_lds_fence();
-#pragma unroll
-    for (int j = 0; j < MM; ++j) {
-        const int c = a + A * j;
-        cpx acc = exch[c * PS + r];
-#pragma unroll
-        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[c * PS + 16 * ap + r], wsm[(ap * c) % L]);
-        out[j] = acc;
-    }
+    wide_forward_finish<L>(g, exch, LdsPow{ wsm }, t, out);
 }
-
 // c[mm] = mode t + L mm of the row. On return y[i] = sample t + L i.
-// Lane l = (t1 = l % Q, rq = l / Q), Q = L / 4, forms the first-pass inputs of the four lanes t1 + Q t2 for the bins
-// r = rq + 4 ri (wide_backward_partial_tw) and parks them for their owners at [r][lane ^ (Q rq)], rows of L: the owners
-// read a row as L consecutive elements, and the XOR puts the four rq of one write Q elements apart, so that the 32
-// lanes of a half wavefront hit 32 different bank pairs in both directions.
 template <int L>
 TFNO_DEV void wide_rows_backward(const cpx (&c)[64 / L], const cpx* twrow, const cpx* wsm, cpx* exch, int t, cpx (&y)[16])
 {
-    constexpr int Q = L / 4;
-    static_assert(16 * L <= L * 17, "the parked values fit the group's region");
-    wave_lds_fence();
-#pragma unroll
-    for (int mm = 0; mm < 64 / L; ++mm) exch[t + L * mm] = c[mm];
-    wave_lds_fence();
-    cpx part[16];
-    const int t1 = t % Q, rq = t / Q;
-    wide_backward_partial_tw<L>(exch, 1, t, wsm[t1], wsm[2 * t1], wsm[3 * t1], part);
-    wave_lds_fence();                                // every lane of the group has read the 64 modes
-#pragma unroll
-    for (int ri = 0; ri < 4; ++ri)
-#pragma unroll
-        for (int t2 = 0; t2 < 4; ++t2) exch[(rq + 4 * ri) * L + t1 + Q * (t2 ^ rq)] = part[4 * ri + t2];
-    wave_lds_fence();
     cpx e[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) e[r] = exch[r * L + (t ^ (Q * (r & 3)))];
+    wide_backward_inputs<L>(c, LdsPow{ wsm }, exch, t, e);
     inv_pass2_lds(e, twrow, y);
 }
 
