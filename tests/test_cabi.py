@@ -46,6 +46,16 @@ def test_codelets_on_cpu(tmp_path):
     assert out.strip().endswith("OK"), out
 
 
+def test_group_transforms_with_their_exchange_layouts_on_cpu(tmp_path):
+    """the device functions of group_fft.h, one host thread per lane and a barrier where the wavefront runs in lockstep:
+    lengths 128 to 1024 forward and backward through the real LDS layouts, against a double-precision DFT"""
+    exe = str(tmp_path / "group_lanes_check")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-pthread", os.path.join(ROOT, "tests", "host", "group_lanes_check.cpp"), "-o", exe],
+                   check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=300).stdout
+    assert out.strip().endswith("OK"), out
+
+
 def test_cmake_package_builds_and_links(tmp_path):
     """the CMake side of the integration: the top-level CMakeLists.txt builds libturbofno.so for gfx950 (library target
     only), installs it with its package file, and a consumer that says find_package(turbofno) +

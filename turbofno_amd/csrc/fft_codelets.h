@@ -407,6 +407,10 @@ TFNO_DEV void wave_lds_fence()
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+#else
+// Host builds (CPU checks of the group transforms): the lanes of a group are threads there, and the check supplies
+// the point at which all of them have arrived.
+void wave_lds_fence();
 #endif
 
 }  // namespace tfno

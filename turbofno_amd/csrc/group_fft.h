@@ -28,10 +28,16 @@ template <int LOGDY> struct Geo1D {
 //     covers 32 consecutive elements per half wavefront, the write of one bin is conflict-free for L = 32 (2-way for 64);
 //   second exchange: [c][16 a' + r] with a pitch of L + 16: writes are consecutive, and the lanes a and a + 1 of a half
 //     wavefront, which read the rows c = a + A j and c + 1, land 16 elements apart modulo 32.
-// wpow(e) = w_L^e, e < L: from the constant table, or from LDS where a global load would be in the way.
+// The powers w_L^e, e < L, come from the constant table, or (FROM_ARRAY) from an array of L values that the caller keeps
+// in LDS where a global load would be in the way.
 // g[]: first-pass results, already twiddled. On return out[j] = mode t + L j.
-template <int L, class Pow>
-TFNO_DEV void wide_forward_finish(const cpx (&g)[16], cpx* exch, Pow wpow, int t, cpx (&out)[64 / L])
+template <int L, bool FROM_ARRAY> TFNO_DEV cpx wide_pow(const cpx* powers, int e)
+{
+    if constexpr (FROM_ARRAY) return powers[e];
+    else return kTwiddle1024[(e * (1024 / L)) & 1023];
+}
+template <int L, bool FROM_ARRAY>
+TFNO_DEV void wide_forward_finish(const cpx (&g)[16], cpx* exch, const cpx* powers, int t, cpx (&out)[64 / L])
 {
     constexpr int A = L / 16, MM = 64 / L, P1 = 16 * A + 1, PS = L + 16;
     static_assert(16 * P1 <= L * 17 && 4 * PS <= L * 17, "both exchanges fit the group's region");
@@ -56,7 +62,7 @@ TFNO_DEV void wide_forward_finish(const cpx (&g)[16], cpx* exch, Pow wpow, int t
         const int c = a + A * j;
         cpx acc = exch[c * PS + r];
 #pragma unroll
-        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[c * PS + 16 * ap + r], wpow((ap * c) % L));
+        for (int ap = 1; ap < A; ++ap) cfma(acc, exch[c * PS + 16 * ap + r], wide_pow<L, FROM_ARRAY>(powers, (ap * c) % L));
         out[j] = acc;
     }
 }
@@ -66,8 +72,8 @@ TFNO_DEV void wide_forward_finish(const cpx (&g)[16], cpx* exch, Pow wpow, int t
 // t1 + Q t2 for the bins r = rq + 4 ri (wide_backward_partial_tw) and parks them for their owners at
 // [r][lane ^ (Q rq)], rows of L: the owners read a row as L consecutive elements, and the XOR puts the four rq of one
 // write Q elements apart, so that the 32 lanes of a half wavefront hit 32 different bank pairs in both directions.
-template <int L, class Pow>
-TFNO_DEV void wide_backward_inputs(const cpx (&c)[64 / L], Pow wpow, cpx* exch, int t, cpx (&e)[16])
+template <int L, bool FROM_ARRAY>
+TFNO_DEV void wide_backward_inputs(const cpx (&c)[64 / L], const cpx* powers, cpx* exch, int t, cpx (&e)[16])
 {
     constexpr int Q = L / 4;
     wave_lds_fence();
@@ -76,7 +82,8 @@ TFNO_DEV void wide_backward_inputs(const cpx (&c)[64 / L], Pow wpow, cpx* exch, 
     wave_lds_fence();
     cpx part[16];
     const int t1 = t % Q, rq = t / Q;
-    wide_backward_partial_tw<L>(exch, 1, t, wpow(t1), wpow(2 * t1), wpow(3 * t1), part);
+    wide_backward_partial_tw<L>(exch, 1, t, wide_pow<L, FROM_ARRAY>(powers, t1), wide_pow<L, FROM_ARRAY>(powers, 2 * t1),
+                                wide_pow<L, FROM_ARRAY>(powers, 3 * t1), part);
     wave_lds_fence();                                // every lane of the group has read the 64 modes
 #pragma unroll
     for (int ri = 0; ri < 4; ++ri)
@@ -86,14 +93,6 @@ TFNO_DEV void wide_backward_inputs(const cpx (&c)[64 / L], Pow wpow, cpx* exch, 
 #pragma unroll
     for (int r = 0; r < 16; ++r) e[r] = exch[r * L + (t ^ (Q * (r & 3)))];
 }
-template <int L> struct TablePow {                   // w_L^e from the constant table
-    TFNO_DEV cpx operator()(int e) const { return kTwiddle1024[(e * (1024 / L)) & 1023]; }
-};
-struct LdsPow {                                      // from an LDS array of the L powers
-    const cpx* w;
-    TFNO_DEV cpx operator()(int e) const { return w[e]; }
-};
-
 // Mode that lane t of an L-lane group holds in out[mm] after a forward transform.
 template <int LOGDY> TFNO_DEV constexpr int forward_mode_of_lane(int t, int mm)
 {
@@ -109,7 +108,7 @@ TFNO_DEV void group_forward_finish(const cpx (&g)[16], cpx* exch, int t, cpx (&o
 {
     constexpr int L = Geo1D<LOGDY>::L;
     if constexpr (L >= 32) {
-        wide_forward_finish<L>(g, exch, TablePow<L>{}, t, out);
+        wide_forward_finish<L, false>(g, exch, nullptr, t, out);
         return;
     }
     wave_lds_fence();
@@ -149,7 +148,7 @@ TFNO_DEV void group_backward(const cpx (&c)[Geo1D<LOGDY>::MM], const cpx (&tw)[1
     constexpr int L = Geo1D<LOGDY>::L;
     cpx e[16];
     if constexpr (L >= 32) {
-        wide_backward_inputs<L>(c, TablePow<L>{}, exch, t, e);
+        wide_backward_inputs<L, false>(c, nullptr, exch, t, e);
     } else {
         wave_lds_fence();
         if constexpr (L == 16) {
@@ -252,14 +251,14 @@ TFNO_DEV void rows128_backward(const cpx (&c)[8], const TW& twrow, cpx* exch, in
 template <int L>
 TFNO_DEV void wide_rows_forward_finish(const cpx (&g)[16], cpx* exch, const cpx* wsm, int t, cpx (&out)[64 / L])
 {
-    wide_forward_finish<L>(g, exch, LdsPow{ wsm }, t, out);
+    wide_forward_finish<L, true>(g, exch, wsm, t, out);
 }
 // c[mm] = mode t + L mm of the row. On return y[i] = sample t + L i.
 template <int L>
 TFNO_DEV void wide_rows_backward(const cpx (&c)[64 / L], const cpx* twrow, const cpx* wsm, cpx* exch, int t, cpx (&y)[16])
 {
     cpx e[16];
-    wide_backward_inputs<L>(c, LdsPow{ wsm }, exch, t, e);
+    wide_backward_inputs<L, true>(c, wsm, exch, t, e);
     inv_pass2_lds(e, twrow, y);
 }
 
