@@ -212,6 +212,24 @@ def main():
                         "GBps": round(b1d / (t1d * 1e-3) / 1e9, 1), "hbm_frac": round(b1d / (t1d * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                         "contraction_TFLOPs": round(f1d / (t1d * 1e-3) / 1e12, 2), "fp32_mfma_peak_TFLOPs": 157.3}
 
+    # ---- lengths above 256 (informational): 16 images of 512 x 512, K=32, N=64 on the whole-image kernels (rows of 512 with
+    # 32 lanes each, the 512 rows as two interleaved parts of 256 that the contraction sums over) and in three stages ----
+    long_axes = None
+    if not args.no_comparators:
+        lbs, LD, LK, LN = 16, 512, 32, 64
+        xl = torch.randn((LK, lbs, LD, LD), dtype=torch.complex64, device=dev)
+        Wl = torch.randn((LN, LK), dtype=torch.complex64, device=dev)
+        yl = torch.empty((LN, lbs, LD, LD), dtype=torch.complex64, device=dev)
+        lbytes = 8 * lbs * LD * LD * (LK + LN) + 8 * LK * LN
+        long_axes = {"workload": "2D bs=16 512x512 K=32 N=64", "auto": tf.query_2d_algo(lbs, LD, LD, LK, LN), "algorithmic_bytes": lbytes}
+        for name, a in (("whole_image", tf.ALGO_WHOLE_IMAGE), ("rows_first", tf.ALGO_ROWS_FIRST), ("x_axis_first", tf.ALGO_THREE_KERNEL)):
+            wsl = torch.empty(tf.layer_2d_workspace_bytes(lbs, LD, LD, LK, LN, a), dtype=torch.uint8, device=dev)
+            t = timed(lambda: tf.layer_2d(xl, Wl, y=yl, alpha=1.0, workspace=wsl, algo=a), 10)
+            long_axes[name + "_ms"] = round(t, 4)
+            long_axes[name + "_hbm_frac"] = round(lbytes / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            del wsl
+        del xl, yl
+
     # ---- CPU baseline: fp32 OpenMP restatement of the library baseline, bounded sample -------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -251,6 +269,7 @@ def main():
         "layer_hbm_frac_sync_protocol": round(layer_bytes / (ms_sync * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "stage_ms": {k: round(v, 4) for k, v in stages.items()},
         "roofline": roofline, "cpu_baseline": cpu, "comparators": comparators, "large_hidden_1d": large_hidden,
+        "long_axes_2d": long_axes,
     }
     print(json.dumps(out))
 
