@@ -27,9 +27,13 @@ constexpr int kWGroup = 1032;
 // HBM peak, S = 4096 0.61, S = 3584 0.70). For these strides XCD j walks the j-th eighth of the signal sets instead
 // (tiles of a signal set on consecutive blocks of that XCD): S = 2048 0.65, S = 4096 0.71; up to -26 % at DY = 512.
 // Up to a stride of 16 MiB; beyond it the grids are large enough to hide the effect and the contiguous walk costs 2-5 %.
-// Only for launches that stream x from and y to HBM (`streamed`): as the middle stage of a 2D pipeline, with its input
-// and output in the caches, the same kernels are a quarter SLOWER in that order (16 images of 512 x 512: layer 750 ->
-// 778 us), and keep the interleaved one.
+// Only for launches that stream x from and y to HBM (`streamed`). As the middle stage of a 2D pipeline the kernel itself
+// is faster in that order as well (16 images of 512 x 512, X axis first: 100 -> 94 us, half the tag and write stalls in
+// L2 at the same hit rate), but the backward kernel that follows loses twice as much (472 -> 487 us): it reads the
+// intermediate in its own order and finds less of it still in the Infinity Cache when the eighths were written side by
+// side (its read latency at the memory side rises from 1880 to 2000 cycles, the request counts stay the same). The
+// layer is what counts, so the middle stage keeps the interleaved order. (-DTFNO_MIDDLE_STAGE_WALKS_EIGHTHS builds the
+// other order for measurements.)
 // Workgroup b of a one-dimensional grid runs on XCD b mod 8: renumbered like this, XCD j takes the j-th eighth of n
 // work items, in order, instead of every eighth item.
 __device__ __forceinline__ long xcd_contiguous(long b, long n) { return (n & 7) == 0 ? (b & 7) * (n >> 3) + (b >> 3) : b; }
@@ -40,6 +44,9 @@ __host__ __device__ __forceinline__ bool xcd_walks_an_eighth_1d(long S, int DY)
 }
 __device__ __forceinline__ void decode_block_1d(long S, int ntiles, int DY, bool streamed, long& s, int& tile)
 {
+#ifdef TFNO_MIDDLE_STAGE_WALKS_EIGHTHS
+    streamed = true;
+#endif
     if (streamed && xcd_walks_an_eighth_1d(S, DY)) {
         const long id = blockIdx.x, q = id >> 3;
         s = (id & 7) * (S / 8) + q / ntiles;
