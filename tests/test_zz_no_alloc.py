@@ -33,6 +33,24 @@ def test_noalloc_matches_workspace_entry_point_twice(algo, tol):
         assert rel_l2(got, ref) <= tol["l2"] and max_rel(got, ref) <= tol["max"]
 
 
+def test_noalloc_long_axes_on_the_whole_image_kernels_twice(tol):
+    """lengths above 256 through the whole-image kernels with their intermediates in the static scratch (the spectra of the
+    interleaved parts of every image, then one spectrum per output image): bit-identical to the workspace entry point,
+    second call smaller"""
+    for call, (bs, DX, DY, K, N) in enumerate([(2, 512, 512, 16, 64), (1, 1024, 256, 8, 64)]):
+        print("noalloc long axes call", call, bs, DX, DY, K, N, flush=True)
+        x_h, W_h = workloads.uniform_2d(660 + call, bs, DX, DY, K, N)
+        x, W = torch.from_numpy(x_h).cuda(), torch.from_numpy(W_h).cuda()
+        y_ref = tf.layer_2d(x, W, alpha=1 - 1j, algo=2)
+        y = torch.full((N, bs, DX, DY), complex(np.nan, np.nan), dtype=torch.complex64, device="cuda")
+        tf.layer_2d_noalloc(x, W, y, alpha=1 - 1j, algo=2)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.float32), y_ref.view(torch.float32)), "outputs differ from turbofno_layer_2d"
+        ref = oracle.layer_2d(np.ascontiguousarray(x_h[:, :1]), W_h, 1 - 1j)
+        got = y[:, :1].cpu().numpy()
+        assert rel_l2(got, ref) <= tol["l2"] and max_rel(got, ref) <= tol["max"]
+
+
 @pytest.mark.parametrize("algo", [1, 0])
 def test_noalloc_leaves_the_free_device_memory_unchanged_on_a_fresh_stream(algo, tol):
     """bs = 1, 256 x 256, K = N = 64 runs three kernels whose middle stage (S = 64 signal sets, 64 channels) is the shape
