@@ -1,4 +1,6 @@
-// Whole-image 2D spectral layer (the MI355X-first path of the 2D layer), DX, DY in {128, 256}.
+// Whole-image 2D spectral layer (the MI355X-first path of the 2D layer): images of DX x DY with DX in {128, 256} rows
+// per block - 512 and 1024 rows as two and four interleaved parts of 256 ("decimated images" below) - and rows of DY in
+// {128, 256, 512, 1024}.
 //
 // The reference's "fully fused" 2D variant is three kernels with two HBM round trips of
 // half-truncated intermediates (fusion_variants/2D_D_exp_fused_fft_cgemm_ifft/fused_trunc_2D.cu:150-172:
@@ -28,7 +30,8 @@ constexpr int EXCH_ELEMS = 1024 * 17;            // exchange regions of all lane
 
 // Geometry of the whole-image kernels for a DX x DY image (DX rows of DY contiguous samples).
 // Rows of 256: a 16-lane group owns one row (16 samples per lane). Rows of 128 ("paired"): a 16-lane group owns
-// two rows, 8 samples per lane each, so that a group still covers 128 contiguous bytes per access.
+// two rows, 8 samples per lane each, so that a group still covers 128 contiguous bytes per access. Rows of 512 / 1024
+// ("wide"): a group of 32 / 64 lanes owns one row, 16 samples per lane, 256 / 512 contiguous bytes per access.
 template <int LOGX, int LOGY> struct Geo2D {
     static constexpr int DX = 1 << LOGX, DY = 1 << LOGY;
     static constexpr bool PAIRED = LOGY == 7;
@@ -125,6 +128,7 @@ template <int LOGD> __device__ __forceinline__ void fill_decimation_twiddles(flo
 // Each group keeps ONE row in flight: the loads of its next row are issued as soon as the first radix-4
 // stage has consumed the row registers, so they travel while the rest of the transform runs, across the
 // column pass and across image boundaries. Inter-pass twiddles live in LDS to stay within 128 VGPRs.
+// nimg counts block-images: the 2^LOGR parts of each of the nfull whole images (nimg = nfull when LOGR = 0).
 template <int LOGX, int LOGY, int LOGR>
 __global__ __launch_bounds__(1024) void fft2d_trunc_kernel(const float2* __restrict__ x, float2* __restrict__ spec,
                                                            int nimg, int nfull)
