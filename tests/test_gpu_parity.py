@@ -190,6 +190,29 @@ def test_layer_2d_random_shapes(seed, tol):
     check(y, oracle.layer_2d(x, W, alpha), tol, "layer_2d random %d" % seed)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_layer_2d_random_long_shapes(seed, tol):
+    """seeded random 2D shapes with at least one axis of 512 or 1024, through every algorithm: the three-stage paths and
+    the whole-image kernels with their interleaved parts (DX above 256) and their 32- / 64-lane rows (DY above 256);
+    first batch element against the oracle"""
+    rng = np.random.default_rng(3000 + seed)
+    lengths = [128, 256, 512, 1024]
+    while True:
+        DX, DY = int(rng.choice(lengths)), int(rng.choice(lengths))
+        if max(DX, DY) > 256 and DX * DY <= 512 * 1024:
+            break
+    K = 8 * int(rng.integers(1, 6))
+    N = 64 * int(rng.integers(1, 3))
+    bs = int(rng.integers(1, 4))
+    algo = (2, 2, 1, 3, 0, 2)[seed % 6]
+    alpha = complex(rng.uniform(-1, 1), rng.uniform(-1, 1))
+    print("case layer_2d random long", seed, "bs", bs, DX, DY, "K", K, "N", N, "algo", algo, flush=True)
+    x, W = workloads.uniform_2d(seed, bs, DX, DY, K, N)
+    y = tf.layer_2d(dev(x), dev(W), alpha=alpha, algo=algo)
+    torch.cuda.synchronize()
+    check(y[:, :1], oracle.layer_2d(np.ascontiguousarray(x[:, :1]), W, alpha), tol, "layer_2d random long %d" % seed)
+
+
 def test_layer_2d_closed_forms(tol):
     """impulse and in-band tone through the whole-image path (analytic expectations, no oracle)."""
     K, bs, D, N = 8, 1, 256, 64
