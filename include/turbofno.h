@@ -106,7 +106,8 @@ int turbofno_layer_2d(int bs, int DX, int DY, int K, int N, const void* x, const
  *   turbofno_ifft2d_pad  : spec[nimg][4096] -> y[nimg][DX][DY]  zero-padded 2D backward transform per image
  * The 4096 retained modes of an image are stored in an order private to these two kernels (element
  * mm*(4*DX) + q*(DX/16) + t holds mode (p = t + (DX/16)*mm, q)); a GEMM over the channel dimension does
- * not care. Requires DX, DY in {128, 256}.
+ * not care. Requires DX in {128, 256} and DY in {128, 256, 512, 1024} (the layer handles longer DX as interleaved
+ * parts, which have no stand-alone meaning).
  *   turbofno_cgemm : C[m + n*M] = alpha * sum_k A[m + k*M] * B[k + n*K] + beta * C[m + n*M] (column major,
  *   lda = M, ldb = K, ldc = M) on the fp32 matrix cores. Replaces the reference's cgemm kernel
  *   (fusion_variants/1D_A_exp_fft+cgemm+ifft/cgemm.cuh:4, launch 1D_A.../fused.cu:199), same argument order

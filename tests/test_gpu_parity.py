@@ -284,7 +284,7 @@ def test_unfused_and_half_fused_stages(S, DY, K, N, tol):
     check(y, ref, tol, "fused_cgemm_ifft")
 
 
-@pytest.mark.parametrize("DX,DY", [(256, 256), (128, 256), (256, 128), (128, 128)])
+@pytest.mark.parametrize("DX,DY", [(256, 256), (128, 256), (256, 128), (128, 128), (256, 512), (128, 1024)])
 def test_image_stage_entry_points(DX, DY, tol):
     """turbofno_fft2d_trunc / turbofno_ifft2d_pad on their own, through the documented order of the 4096 retained
     modes: element mm*(64*LX) + q*LX + t holds mode (p = t + LX*mm, q), LX = DX/16"""

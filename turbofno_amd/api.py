@@ -286,7 +286,8 @@ def layer_2d_noalloc(x, W, y, alpha=1.0 + 0j, algo=0):
 
 
 def fft2d_trunc(x, spec):
-    """x: [nimg][DX][DY], DX, DY in {128, 256} -> spec: [nimg][4096] (retained 64 x 64 modes, kernel-private order)."""
+    """x: [nimg][DX][DY], DX in {128, 256}, DY in {128, 256, 512, 1024} -> spec: [nimg][4096] (retained 64 x 64 modes,
+    kernel-private order)."""
     _need(x.dim() >= 2, "x must end in [DX][DY]")
     nimg = x.numel() // (x.shape[-1] * x.shape[-2])
     _need(nimg > 0, "x holds no image")

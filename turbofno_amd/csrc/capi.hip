@@ -34,7 +34,7 @@ int log2_exact(long v)
 }
 
 bool length_built(int logD) { return logD >= 7 && logD <= 10; }          // 1D kernels and the X-axis kernels
-bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // whole-image 2D kernels, one block per image
+bool image_length_built(int logD) { return logD == 7 || logD == 8; }    // rows of an image that one block holds
 // the whole-image path of the 2D layer also takes DX of 512 and 1024, as two or four decimated parts of 256 rows
 bool whole_image_built(int DX, int DY) { return length_built(log2_exact(DX)) && length_built(log2_exact(DY)); }
 int image_parts(int DX) { return DX > 256 ? DX / 256 : 1; }
@@ -226,8 +226,8 @@ int turbofno_fft2d_trunc(int DX, int DY, const void* x, void* spec, long nimg, v
     if (!x || !spec) return fail(TURBOFNO_ERR_INVALID_ARG, "x and spec must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
     const int logDX = log2_exact(DX), logDY = log2_exact(DY);
-    if (!image_length_built(logDX) || !image_length_built(logDY))
-        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
+    if (!image_length_built(logDX) || !length_built(logDY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the stand-alone image transforms are built for DX in {128, 256} and DY in {128, 256, 512, 1024}", DX, DY);
     return hip_status(tfno::launch_fft2d_trunc(logDX, logDY, (const float2*)x, (float2*)spec, nimg, (hipStream_t)stream), "fft2d_trunc launch");
 }
 
@@ -236,8 +236,8 @@ int turbofno_ifft2d_pad(int DX, int DY, const void* spec, void* y, long nimg, vo
     if (!spec || !y) return fail(TURBOFNO_ERR_INVALID_ARG, "spec and y must be non-null device pointers");
     if (nimg <= 0 || nimg > 0x7fffffffL) return fail(TURBOFNO_ERR_INVALID_ARG, "nimg=%ld out of range", nimg);
     const int logDX = log2_exact(DX), logDY = log2_exact(DY);
-    if (!image_length_built(logDX) || !image_length_built(logDY))
-        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: whole-image transforms are built for lengths in {128, 256}", DX, DY);
+    if (!image_length_built(logDX) || !length_built(logDY))
+        return fail(TURBOFNO_ERR_UNSUPPORTED, "DX=%d, DY=%d: the stand-alone image transforms are built for DX in {128, 256} and DY in {128, 256, 512, 1024}", DX, DY);
     return hip_status(tfno::launch_ifft2d_pad(logDX, logDY, (const float2*)spec, (float2*)y, nimg, (hipStream_t)stream), "ifft2d_pad launch");
 }
 
